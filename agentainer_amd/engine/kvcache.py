@@ -46,6 +46,9 @@ class KVCheckpoint:
     length: int
     n_pages: int
     data: torch.Tensor  # pinned host [n_layers, n_pages, page_shorts] bf16
+    # per-sequence recurrent state (layouts that keep one): host fp32
+    # [n_layers, state_elems]
+    state: Optional[torch.Tensor] = None
 
 
 class GQALayout:
@@ -141,6 +144,98 @@ class HeadKVLayout:
             -1, *entry[1].shape[1:]))
 
 
+class HybridStateLayout:
+    """Layers that cache per-token K/V pages, per-SEQUENCE state, or both.
+
+    kv_shapes[l] is (kv_heads, key_dim, value_dim) — pools as in
+    HeadKVLayout — or None for a layer without attention. state_shapes[l]
+    maps a name to the shape of one sequence's fp32 state tensor of that
+    layer (a recurrent memory, the tail of a short convolution); the
+    manager allocates each as [slots, *shape], indexed by the sequence
+    slot, so a sequence's state is addressed on the device by the same
+    number as its page-table row. The kernels treat a sequence that
+    starts at position 0 as having zero state, so a slot needs no
+    clearing when it is handed to the next sequence."""
+
+    def __init__(self, kv_shapes, state_shapes):
+        self.kv_shapes = [None if s is None else tuple(int(v) for v in s)
+                          for s in kv_shapes]
+        self.state_shapes = [{k: tuple(int(x) for x in v)
+                              for k, v in d.items()} for d in state_shapes]
+        assert len(self.kv_shapes) == len(self.state_shapes)
+        self.n_layers = len(self.kv_shapes)
+
+    def alloc(self, n_pages, page_size, device, dtype):
+        out = []
+        for s in self.kv_shapes:
+            if s is None:
+                out.append((None, None))
+            else:
+                g, d, dv = s
+                out.append((torch.zeros(n_pages, g, page_size, d, dtype=dtype,
+                                        device=device),
+                            torch.zeros(n_pages, g, page_size, dv, dtype=dtype,
+                                        device=device)))
+        return out
+
+    def alloc_state(self, n_slots, device):
+        return [{k: torch.zeros(n_slots, *shape, dtype=torch.float32,
+                                device=device) for k, shape in d.items()}
+                for d in self.state_shapes]
+
+    def page_elems(self, page_size: int) -> int:
+        return max([g * (d + dv) for g, d, dv in
+                    (s for s in self.kv_shapes if s is not None)] + [1]
+                   ) * page_size
+
+    def state_elems(self) -> int:
+        """fp32 values of one sequence's state in the largest layer."""
+        n = 0
+        for d in self.state_shapes:
+            tot = 0
+            for shape in d.values():
+                e = 1
+                for x in shape:
+                    e *= x
+                tot += e
+            n = max(n, tot)
+        return n
+
+    def state_bytes_per_seq(self) -> int:
+        tot = 0
+        for d in self.state_shapes:
+            for shape in d.values():
+                e = 4
+                for x in shape:
+                    e *= x
+                tot += e
+        return tot
+
+    def gather(self, entry, staging, page_ids):
+        if entry[0] is not None:
+            HeadKVLayout.gather(self, entry, staging, page_ids)
+
+    def scatter(self, entry, staging, page_ids):
+        if entry[0] is not None:
+            HeadKVLayout.scatter(self, entry, staging, page_ids)
+
+    def gather_state(self, state, slot: int, row: torch.Tensor) -> None:
+        """One layer's state of `slot` -> flat fp32 row."""
+        off = 0
+        for k in sorted(state):
+            t = state[k][slot].reshape(-1)
+            row[off:off + t.numel()] = t
+            off += t.numel()
+
+    def scatter_state(self, state, slot: int, row: torch.Tensor) -> None:
+        off = 0
+        for k in sorted(state):
+            n = state[k][slot].numel()
+            state[k][slot] = row[off:off + n].view(state[k].shape[1:]).to(
+                state[k].device)
+            off += n
+
+
 class KVCacheManager:
     def __init__(self, n_layers: int, n_kv: int, head_dim: int, page_size: int,
                  n_pages: int, device="cpu", dtype=torch.bfloat16,
@@ -160,6 +255,10 @@ class KVCacheManager:
         # scale-free semantics (e4m3 range +-448 covers post-norm K/V)
         self.dtype = dtype
         self.caches = self.layout.alloc(n_pages, page_size, device, dtype)
+        # per-sequence-slot state (recurrent memories, convolution tails)
+        # of layouts that keep one: per layer a dict name -> [slots, ...]
+        self.states = (self.layout.alloc_state(max_slots, device)
+                       if hasattr(self.layout, "alloc_state") else None)
         if isinstance(self.layout, GQALayout):
             self.k_caches: List[torch.Tensor] = [c[0] for c in self.caches]
             self.v_caches: List[torch.Tensor] = [c[1] for c in self.caches]
@@ -214,6 +313,11 @@ class KVCacheManager:
         return self.n_pages - self.free_pages
 
     def kv_caches(self) -> List[Tuple[torch.Tensor, torch.Tensor]]:
+        """Per layer what the model's forward reads and writes: the page
+        pools, followed by the layer's state dict where the layout keeps
+        per-sequence state."""
+        if self.states is not None:
+            return [tuple(c) + (st,) for c, st in zip(self.caches, self.states)]
         return list(self.caches)
 
     def has_seq(self, seq_id: str) -> bool:
@@ -231,7 +335,7 @@ class KVCacheManager:
             if not s:
                 return 0
             return (len(s.pages) * self.page_shorts * self.n_layers *
-                    self.caches[0][0].element_size())
+                    torch.empty(0, dtype=self.dtype).element_size())
 
     # ---------- allocation ----------
 
@@ -499,7 +603,17 @@ class KVCacheManager:
                 return None
             pages = list(s.pages)
             length = s.length
+            slot = self._slot_of[seq_id]
         n = len(pages)
+        state = None
+        if self.states is not None:
+            state = torch.zeros(self.n_layers, self.layout.state_elems(),
+                                dtype=torch.float32)
+            for li in range(self.n_layers):
+                row = torch.zeros(state.size(1), dtype=torch.float32,
+                                  device=self.device)
+                self.layout.gather_state(self.states[li], slot, row)
+                state[li].copy_(row)
         page_ids = torch.tensor(pages, dtype=torch.int32, device=self.device)
         is_gpu = str(self.device) not in ("cpu",)
         host = torch.empty(self.n_layers, n, self.page_shorts, dtype=self.dtype,
@@ -518,7 +632,7 @@ class KVCacheManager:
                 host[li].copy_(staging)
         if free:
             self.free_seq(seq_id)
-        return KVCheckpoint(length=length, n_pages=n, data=host)
+        return KVCheckpoint(length=length, n_pages=n, data=host, state=state)
 
     def restore(self, seq_id: str, ckpt: Optional[KVCheckpoint]) -> None:
         """Upload a checkpoint into freshly allocated pages."""
@@ -533,6 +647,11 @@ class KVCacheManager:
             s.pages = [self._free.pop() for _ in range(ckpt.n_pages)]
             s.length = ckpt.length
             pages = list(s.pages)
+            slot = self._slot_of[seq_id]
+        if self.states is not None and ckpt.state is not None:
+            for li in range(self.n_layers):
+                self.layout.scatter_state(self.states[li], slot,
+                                          ckpt.state[li].to(self.device))
         page_ids = torch.tensor(pages, dtype=torch.int32, device=self.device)
         is_gpu = str(self.device) not in ("cpu",)
         for li in range(self.n_layers):

@@ -278,6 +278,15 @@ class ModelInstance:
         # needs no cross-rank traffic.
         self.async_decode = ((self.use_graph or self._emulate_dev)
                              and bool(engine_cfg.get("async_decode", True)))
+        # models that carry per-sequence recurrent state: a state cannot
+        # be un-stepped, so the speculative decode step (which appends a
+        # token that may have to be rolled back) is off, and a sequence
+        # cannot adopt another one's pages without the state that belongs
+        # to the end of the shared prefix, so prefix sharing is off too
+        self.stateful = self.kvm.states is not None
+        if self.stateful:
+            self.async_decode = False
+            self.prefix_sharing = False
         # index of this model in the engine's creation order — the wire
         # identity in binary step plans (identical on every TP rank)
         self._model_idx = 0
@@ -326,11 +335,17 @@ class ModelInstance:
         eb = 1 if str(engine_cfg.get("kv_dtype", "bf16")).startswith(("fp8", "e4m3")) else 2
         if str(engine_cfg.get("dtype", "bf16")) in ("fp32", "float32"):
             eb = 4
-        bytes_per_page = cfg.kv_bytes_per_token(eb) * page_size // max(tp_size, 1)
+        bytes_per_page = max(
+            cfg.kv_bytes_per_token(eb) * page_size // max(tp_size, 1), 1)
         pool_gb = float(engine_cfg.get("kv_pool_gb", 0.0))
         if device.startswith("cuda") and pool_gb <= 0:
             free, _total = torch.cuda.mem_get_info()
             pool_bytes = int(free * 0.80)  # leave headroom for activations
+            if hasattr(cfg, "state_bytes_per_seq"):
+                # per-sequence recurrent state is allocated for every slot
+                pool_bytes = max(pool_bytes - cfg.state_bytes_per_seq()
+                                 * int(engine_cfg.get("max_seqs", 2048)),
+                                 pool_bytes // 8)
         elif pool_gb > 0:
             pool_bytes = int(pool_gb * (1 << 30))
         else:
@@ -925,6 +940,11 @@ class ModelInstance:
         page_table = self.kvm.page_table(seq_ids, device="cpu")
         seq_lens = self.kvm.seq_lens(seq_ids, device="cpu")
         n_real = len(seq_ids)
+        # per-sequence state (recurrent layers) is addressed by slot; the
+        # pad row below parks its state on the reserved pad slot
+        state_slots = ([self.kvm.slot(sid) for sid in seq_ids]
+                       if self.stateful else None)
+        pad_state_slot = None
         # pad the token dimension to a bucketed GEMM shape: extra tokens
         # form one fake row whose K/V land in the reserved scratch page 0
         # and whose logits are never read (last_rows covers real rows only)
@@ -937,6 +957,7 @@ class ModelInstance:
             ids.extend([0] * n_pad)
             positions.extend(i % PS for i in range(n_pad))
             slots.extend(i % PS for i in range(n_pad))  # page 0 scratch
+            pad_state_slot = self._pad_slot
             # the attention kernel requires seq_len >= qlen (causal window
             # math); the pad row's "pages" are ceil(n_pad/PS) references to
             # scratch page 0, so its K/V reads stay in-bounds
@@ -962,6 +983,11 @@ class ModelInstance:
             query_lens=torch.tensor(q_lens, dtype=torch.int32, device=dev),
             max_qlen=max(q_lens),
         )
+        if state_slots is not None:
+            if pad_state_slot is not None:
+                state_slots.append(pad_state_slot)
+            md.state_slots = torch.tensor(state_slots, dtype=torch.long,
+                                          device=dev)
         input_ids = torch.tensor(ids, dtype=torch.long, device=dev)
         if want is None:
             rows_l = [s + l - 1
@@ -1032,7 +1058,8 @@ class ModelInstance:
         pages = pt.gather(1, page_idx.unsqueeze(1)).squeeze(1).long()
         slots = pages * PS + (pos % PS).long()             # pad rows -> page 0
         md = AttnMetadata(page_table=pt, seq_lens=lens + 1,
-                          slot_mapping=slots, positions=pos, is_prefill=False)
+                          slot_mapping=slots, positions=pos, is_prefill=False,
+                          state_slots=rows)
         logits = self.model(input_ids, md, self.kvm.kv_caches(), None)
         kvm.dev_seq_lens.index_add_(0, rows, inc)
         kvm.dev_seq_lens.index_fill_(0, self._pad_slot_t, -1)
@@ -1126,6 +1153,10 @@ class ModelInstance:
             positions=torch.tensor(positions, dtype=torch.int32, device=dev),
             is_prefill=False,
         )
+        if self.stateful:
+            md.state_slots = torch.tensor(
+                [self.kvm.slot(sid) for sid in seq_ids], dtype=torch.long,
+                device=dev)
         input_ids = torch.tensor(ids, dtype=torch.long, device=dev)
         return self.model(input_ids, md, self.kvm.kv_caches(), None)
 
@@ -1761,8 +1792,11 @@ class LLMEngine:
         return os.path.join(d, f"{agent_id}{suffix}.pt")
 
     def _save_disk_ckpt(self, agent_id: str, ckpt: KVCheckpoint) -> None:
-        torch.save({"length": ckpt.length, "n_pages": ckpt.n_pages,
-                    "data": ckpt.data.cpu()}, self._ckpt_path(agent_id))
+        d = {"length": ckpt.length, "n_pages": ckpt.n_pages,
+             "data": ckpt.data.cpu()}
+        if ckpt.state is not None:
+            d["state"] = ckpt.state.cpu()
+        torch.save(d, self._ckpt_path(agent_id))
 
     def _load_disk_ckpt(self, agent_id: str) -> Optional[KVCheckpoint]:
         p = self._ckpt_path(agent_id)
@@ -1771,7 +1805,7 @@ class LLMEngine:
         try:
             d = torch.load(p, map_location="cpu", weights_only=True)
             return KVCheckpoint(length=d["length"], n_pages=d["n_pages"],
-                                data=d["data"])
+                                data=d["data"], state=d.get("state"))
         except Exception:
             return None
 

@@ -67,6 +67,9 @@ class AttnMetadata:
     # host-known max(query_lens): avoids a BLOCKING D2H read in the
     # attention launcher (measured ~2 ms/call behind a deep GPU queue)
     max_qlen: int = 0
+    # [B] int64 — each sequence's slot in the cache manager's per-sequence
+    # state tensors (models with recurrent layers); None otherwise
+    state_slots: Optional[torch.Tensor] = None
 
 
 class LlamaAttention(torch.nn.Module):

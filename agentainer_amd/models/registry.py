@@ -18,6 +18,9 @@ FAMILIES: Dict[str, Tuple[str, str, str, str]] = {
                 "make_lelitar_instance", "latent"),
     "Volalorn": ("agentainer_amd.models.volalorn", "VOLALORN_CONFIGS",
                  "make_volalorn_instance", "masked"),
+    # convolved attention reuses the masked-attention kernels
+    "Pekarax": ("agentainer_amd.models.pekarax", "PEKARAX_CONFIGS",
+                "make_pekarax_instance", "masked+recurrent"),
 }
 
 
@@ -59,6 +62,7 @@ def make_instance(arch: str, model: str, device: str, engine_cfg):
 
 
 def build_target(model: str) -> str:
-    """ops.build target holding the kernels `model` runs on."""
+    """ops.build target holding the kernels `model` runs on ("a+b" names
+    several)."""
     arch = family_of(model)
     return FAMILIES[arch][3] if arch else "core"

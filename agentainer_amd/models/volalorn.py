@@ -85,6 +85,10 @@ class MaskedAttentionConfig:
     qkv_bias: bool = False
     norm_first: bool = False  # True: weighted q/k norm, then rotary;
     #                           False: rotary, then weightless unit rms
+    conv_taps: int = 0        # > 0: a depthwise causal convolution over time
+    #                           on the projected q, k, v (before norm and
+    #                           rotary); its last taps-1 inputs are
+    #                           per-sequence state
 
 
 @dataclass
@@ -207,6 +211,9 @@ class MaskedAttention(torch.nn.Module):
         self.k_norm = _param(mc.dim, dtype=f32) if mc.norm_first else None
         self.key_bias = _param(H, dtype=f32) if mc.key_bias else None
         self.w_o = _param(width, H * mc.vdim, dtype=dtype)
+        self.conv_channels = self.q_sz + self.k_sz + self.v_sz
+        self.w_conv = (_param(self.conv_channels, mc.conv_taps, dtype=f32)
+                       if mc.conv_taps > 0 else None)
         freqs, self.rot_amp = ops.rotary_frequencies(
             mc.rot_dims, mc.rot_base, mc.rot_scaling)
         self.register_buffer("rot_freqs", freqs, persistent=False)
@@ -233,6 +240,9 @@ class MaskedAttention(torch.nn.Module):
         if mc.key_bias:
             self.key_bias.copy_(get("pb").float())
         self.w_o.copy_(get("o"))
+        if mc.conv_taps > 0:
+            self.w_conv.copy_(torch.cat(
+                [get("q.conv"), get("k.conv"), get("v.conv")], dim=0).float())
 
     def rotary_key(self):
         """Layers with equal keys share one cos/sin table per step."""
@@ -243,7 +253,10 @@ class MaskedAttention(torch.nn.Module):
 
     def forward(self, h: torch.Tensor, k_cache: torch.Tensor,
                 v_cache: torch.Tensor, md: AttnMetadata,
-                tables: Optional[dict] = None) -> torch.Tensor:
+                tables: Optional[dict] = None,
+                conv_tail: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """conv_tail [slots, taps-1, q+k+v channels] fp32 (the cache
+        manager's per-sequence state) is required when conv_taps > 0."""
         mc = self.mc
         key = self.rotary_key()
         cos_sin = tables.get(key) if tables is not None else None
@@ -256,10 +269,17 @@ class MaskedAttention(torch.nn.Module):
         proj = ops.linear(h, self.w_in, bias=self.b_in)
         k0, v0 = self.q_sz, self.q_sz + self.k_sz
         g0 = v0 + self.v_sz
+        qkv = proj
+        if mc.conv_taps > 0:
+            qkv = torch.empty(T, g0, dtype=h.dtype, device=h.device)
+            ops.short_conv_state(
+                qkv, proj[:, :g0], self.w_conv, conv_tail, md.state_slots,
+                md.seq_lens, md.query_starts if md.is_prefill else None,
+                md.query_lens if md.is_prefill else None)
         # strided views into the GEMM output: the kernels take row strides
-        q = proj[:, :k0].view(T, H, mc.dim)
-        k = proj[:, k0:v0].view(T, G, mc.dim)
-        v = proj[:, v0:g0].view(T, G, mc.vdim)
+        q = qkv[:, :k0].view(T, H, mc.dim)
+        k = qkv[:, k0:v0].view(T, G, mc.dim)
+        v = qkv[:, v0:g0].view(T, G, mc.vdim)
         ops.rotary_norm_append(q, k, v, k_cache, v_cache, cos_sin,
                                md.slot_mapping, self.eps, self.q_norm,
                                self.k_norm, mc.norm_first)

@@ -655,3 +655,145 @@ def masked_attention(out, q, k_cache, v_cache, page_table, seq_lens,
                                    sigmoid_weights, softcap, key_bias,
                                    head_gate)
     return out
+
+
+# ---------------------------------------------------------------------
+# Post-norm residual with (1 + w) RMS norm, short causal convolutions with
+# a per-sequence tail, matrix-memory recurrences (gated linear attention,
+# gated delta rule, mLSTM) over per-sequence state, per-head output norm +
+# gate, group-limited softmax routing and clamped gated experts. Own
+# extension (_hip_recurrent.so), same policy: required on a GPU, fp32
+# torch references on CPU.
+# ---------------------------------------------------------------------
+
+_recurrent = None
+_recurrent_err: Optional[str] = None
+
+
+def _load_recurrent():
+    global _recurrent, _recurrent_err
+    if _recurrent is not None or _recurrent_err is not None:
+        return _recurrent
+    so = os.path.join(os.path.dirname(__file__), "_hip_recurrent.so")
+    if not os.path.exists(so):
+        _recurrent_err = (f"HIP extension not built ({so} missing); run "
+                          "python -m agentainer_amd.ops.build recurrent")
+        return None
+    try:
+        import importlib.util
+
+        spec = importlib.util.spec_from_file_location(
+            "agentainer_amd.ops._hip_recurrent", so)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _recurrent = mod
+    except Exception as exc:  # noqa: BLE001
+        _recurrent_err = f"HIP extension failed to load: {exc}"
+    return _recurrent
+
+
+def recurrent_available() -> bool:
+    return _load_recurrent() is not None
+
+
+def _dispatch_recurrent(name: str, t: torch.Tensor):
+    if t.is_cuda:
+        mod = _load_recurrent()
+        if mod is None:
+            raise RuntimeError(
+                f"op {name!r} on GPU requires the gfx950 HIP extension: "
+                f"{_recurrent_err}")
+        return mod
+    return None
+
+
+SCAN_GLA = reference.SCAN_GLA
+SCAN_DELTA = reference.SCAN_DELTA
+SCAN_MLSTM = reference.SCAN_MLSTM
+
+
+def postln_rmsnorm_residual(x_res, y, w1p, eps: float, h_out,
+                            alpha: float = 1.0, y_scale: float = 1.0,
+                            y2=None, y2_scale: float = 1.0, row_add=None):
+    """x_res(fp32) <- rms_norm((alpha + row_add[t]) * x_res + y_scale * y
+    + y2_scale * y2) * w1p; h_out = x_res in the compute dtype."""
+    mod = _dispatch_recurrent("postln_rmsnorm_residual", x_res)
+    if mod:
+        mod.postln_rmsnorm_residual(x_res, y, float(y_scale), y2,
+                                    float(y2_scale), float(alpha), row_add,
+                                    w1p, float(eps), h_out)
+    else:
+        reference.postln_rmsnorm_residual(x_res, y, y_scale, y2, y2_scale,
+                                          alpha, row_add, w1p, eps, h_out)
+    return h_out
+
+
+def short_conv_state(out, u, w, tail, state_slots, seq_lens, query_starts,
+                     query_lens, silu: bool = False, norm_channels: int = 0,
+                     head_dim: int = 1, lead_channels: int = 0,
+                     lead_scale: float = 1.0, l2_eps: float = 1e-6):
+    mod = _dispatch_recurrent("short_conv_state", u)
+    if mod:
+        mod.short_conv_state(out, u, w, tail, state_slots, seq_lens,
+                             query_starts, query_lens, bool(silu),
+                             int(norm_channels), int(head_dim),
+                             int(lead_channels), float(lead_scale),
+                             float(l2_eps))
+    else:
+        reference.short_conv_state(out, u, w, tail, state_slots, seq_lens,
+                                   query_starts, query_lens, silu,
+                                   norm_channels, head_dim, lead_channels,
+                                   lead_scale, l2_eps)
+    return out
+
+
+def matrix_memory_scan(kind: int, out, q, k, v, gate, gate_bias, head_rate,
+                       beta, q_scale: float, gate_param: float, S, n_state,
+                       m_state, state_slots, seq_lens, query_starts,
+                       query_lens):
+    mod = _dispatch_recurrent("matrix_memory_scan", q)
+    if mod:
+        mod.matrix_memory_scan(int(kind), out, q, k, v, gate, gate_bias,
+                               head_rate, beta, float(q_scale),
+                               float(gate_param), S, n_state, m_state,
+                               state_slots, seq_lens, query_starts,
+                               query_lens)
+    else:
+        reference.matrix_memory_scan(kind, out, q, k, v, gate, gate_bias,
+                                     head_rate, beta, q_scale, gate_param, S,
+                                     n_state, m_state, state_slots, seq_lens,
+                                     query_starts, query_lens)
+    return out
+
+
+def head_rmsnorm_gate(out, o, w, gate, eps: float, silu_gate: bool):
+    mod = _dispatch_recurrent("head_rmsnorm_gate", o)
+    if mod:
+        mod.head_rmsnorm_gate(out, o, w, gate, float(eps), bool(silu_gate))
+    else:
+        reference.head_rmsnorm_gate(out, o, w, gate, eps, silu_gate)
+    return out
+
+
+def grouped_softmax_route(weight, logits, correction, top: int,
+                          n_groups: int, keep_groups: int, scale: float):
+    mod = _dispatch_recurrent("grouped_softmax_route", logits)
+    if mod:
+        mod.grouped_softmax_route(weight, logits, correction, int(top),
+                                  int(n_groups), int(keep_groups),
+                                  float(scale))
+    else:
+        reference.grouped_softmax_route(weight, logits, correction, top,
+                                        n_groups, keep_groups, scale)
+    return weight
+
+
+def routed_clamped_glu(out, gu, weight, n_experts: int, limit: float,
+                       slope: float):
+    mod = _dispatch_recurrent("routed_clamped_glu", gu)
+    if mod:
+        mod.routed_clamped_glu(out, gu, weight, int(n_experts), float(limit),
+                               float(slope))
+    else:
+        reference.routed_clamped_glu(out, gu, weight, n_experts, limit, slope)
+    return out

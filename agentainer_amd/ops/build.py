@@ -48,6 +48,16 @@ MASKED_SOURCES = [
     "masked_attn.hip",
 ]
 
+# post-norm residual, short convolutions with state, matrix-memory scans,
+# head norm + gate, group-limited routing, clamped gated experts
+RECURRENT_SOURCES = [
+    "recurrent_bindings.cpp",
+    "postln_norm.hip",
+    "short_conv.hip",
+    "matrix_memory.hip",
+    "grouped_route.hip",
+]
+
 SOURCES = [
     "bindings.cpp",
     "rmsnorm.hip",
@@ -77,6 +87,11 @@ def _target(target: str):
         return (os.path.join(HERE, f"_hip_masked{sfx}.so"),
                 os.path.join(HERE, "_build_masked" + sfx), MASKED_SOURCES,
                 "_hip_masked")
+    if target == "recurrent":
+        sfx = "_asan" if ASAN else ""
+        return (os.path.join(HERE, f"_hip_recurrent{sfx}.so"),
+                os.path.join(HERE, "_build_recurrent" + sfx),
+                RECURRENT_SOURCES, "_hip_recurrent")
     if target != "core":
         raise ValueError(f"unknown build target {target!r}")
     return OUT, OBJ_DIR, SOURCES, "_hip_ops"
@@ -96,9 +111,12 @@ def needs_build(target: str = "core") -> bool:
 def build(verbose: bool = True, force: bool = False,
           target: str = "core") -> str:
     if target == "all":
-        build(verbose, force, "core")
-        build(verbose, force, "latent")
-        return build(verbose, force, "masked")
+        target = "core+latent+masked+recurrent"
+    if "+" in target:
+        out = ""
+        for t in target.split("+"):
+            out = build(verbose, force, t)
+        return out
     OUT, OBJ_DIR, SOURCES, modname = _target(target)
     if not force and not needs_build(target):
         return OUT

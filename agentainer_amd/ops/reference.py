@@ -502,3 +502,220 @@ def masked_attention(out: torch.Tensor, q: torch.Tensor,
             o = o * torch.sigmoid(head_gate[start:start + qlen].float()
                                   ).unsqueeze(-1)
         out[start:start + qlen] = o.to(out.dtype)
+
+
+# ---------------------------------------------------------------------
+# Post-norm residual with a (1 + w) RMS norm, short causal convolutions
+# with a per-sequence tail, matrix-memory recurrences (gated linear
+# attention, gated delta rule, mLSTM), per-head output norm + gate, and
+# group-limited softmax routing with clamped gated experts.
+# ---------------------------------------------------------------------
+
+def postln_rmsnorm_residual(x_res: torch.Tensor, y, y_scale: float, y2,
+                            y2_scale: float, alpha: float, row_add,
+                            w1p: torch.Tensor, eps: float,
+                            h_out: torch.Tensor) -> None:
+    """s = (alpha + row_add[t]) * x + y_scale * y + y2_scale * y2;
+    x <- s / sqrt(mean(s^2) + eps) * w1p; h_out = x in the compute dtype.
+    x_res is the fp32 residual (rewritten); y, y2, row_add may be None;
+    w1p holds 1 + w."""
+    a = x_res.new_full((x_res.size(0), 1), float(alpha))
+    if row_add is not None:
+        a = a + row_add.float().view(-1, 1)
+    s = x_res * a
+    if y is not None:
+        s = s + y.float() * y_scale
+    if y2 is not None:
+        s = s + y2.float() * y2_scale
+    r = s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps) * w1p.float()
+    x_res.copy_(r)
+    h_out.copy_(r.to(h_out.dtype))
+
+
+def _step_rows(b: int, seq_lens, query_starts, query_lens):
+    """(first row, row count, position of the first row) of sequence b in a
+    step; query_starts / query_lens None = one new token per sequence."""
+    total = int(seq_lens[b])
+    if query_lens is None:
+        return b, 1, total - 1
+    n = int(query_lens[b])
+    return int(query_starts[b]), n, total - n
+
+
+def short_conv_state(out: torch.Tensor, u: torch.Tensor, w: torch.Tensor,
+                     tail: torch.Tensor, state_slots: torch.Tensor,
+                     seq_lens, query_starts, query_lens, silu: bool,
+                     norm_channels: int, head_dim: int, lead_channels: int,
+                     lead_scale: float, l2_eps: float) -> None:
+    """Depthwise causal convolution over time with the last taps-1 inputs
+    of every sequence kept in tail [slots, taps-1, C] (fp32).
+
+    y[t, c] = sum_j w[c, j] * u[t - taps + 1 + j, c]; inputs before this
+    step's rows come from the tail, inputs before position 0 are zero (a
+    sequence whose first row sits at position 0 ignores its tail). Then
+    optionally silu, and for the first norm_channels channels, cut into
+    heads of head_dim, y / sqrt(sum(y^2) + l2_eps); the first lead_channels
+    of those are multiplied by lead_scale. The tail is rewritten."""
+    taps = w.size(1)
+    wf = w.float()
+    for b in range(seq_lens.numel()):
+        s0, n, pos0 = _step_rows(b, seq_lens, query_starts, query_lens)
+        if n <= 0:
+            continue
+        slot = int(state_slots[b])
+        hist = tail[slot].float() if pos0 > 0 else torch.zeros_like(tail[slot])
+        full = torch.cat([hist, u[s0:s0 + n].float()], dim=0)
+        y = torch.zeros(n, u.size(1))
+        for j in range(taps):
+            y = y + wf[:, j] * full[j:j + n]
+        if taps > 1:
+            tail[slot] = full[-(taps - 1):]
+        if silu:
+            y = y * torch.sigmoid(y)
+        if norm_channels > 0:
+            yh = y[:, :norm_channels].reshape(n, -1, head_dim)
+            yh = yh / torch.sqrt(yh.pow(2).sum(-1, keepdim=True) + l2_eps)
+            y[:, :norm_channels] = yh.reshape(n, norm_channels)
+            y[:, :lead_channels] = y[:, :lead_channels] * lead_scale
+        out[s0:s0 + n] = y.to(out.dtype)
+
+
+SCAN_GLA, SCAN_DELTA, SCAN_MLSTM = 0, 1, 2
+
+
+def matrix_memory_scan(kind: int, out: torch.Tensor, q: torch.Tensor,
+                       k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
+                       gate_bias, head_rate, beta, q_scale: float,
+                       gate_param: float, S: torch.Tensor, n_state, m_state,
+                       state_slots: torch.Tensor, seq_lens, query_starts,
+                       query_lens) -> None:
+    """Token-by-token matrix-memory recurrences over per-sequence state.
+
+    q, k [T, G, D]; v [T, H, Dv]; out [T, H, Dv] fp32; head h reads q/k
+    head h // (H/G). S [slots, H, Dv, D] fp32 holds every head's memory
+    transposed (one row per value coordinate). A sequence whose first row
+    sits at position 0 starts from zero state. q is multiplied by q_scale.
+
+    SCAN_GLA:   a = exp(logsigmoid(gate + gate_bias) * gate_param), per key
+                channel (gate [T, H*D]); S <- a S + k v^T; o = S^T q.
+    SCAN_DELTA: g = exp(-exp(head_rate[h]) * softplus(gate + gate_bias)),
+                b = sigmoid(beta[t, h]); S <- g S; u = b (v - S^T k);
+                S <- S + k u^T; o = S^T q.
+    SCAN_MLSTM: gate [T, 2H] = log-input | forget pre-activations,
+                i = c tanh((gate_i + bias_i) / c), f = logsigmoid(c tanh(
+                (gate_f + bias_f) / c)), c = gate_param; m' = max(f + m, i);
+                S <- e^(f+m-m') S + e^(i-m') k v^T, n likewise with k;
+                o = S^T q / (max(|n.q|, e^(-m')) + 1e-6).
+                n_state [slots, H, D], m_state [slots, H]."""
+    H, Dv = v.size(1), v.size(2)
+    G, D = k.size(1), k.size(2)
+    rep = H // G
+    gb = gate_bias.float() if gate_bias is not None else None
+    lsig = torch.nn.functional.logsigmoid
+    for b in range(seq_lens.numel()):
+        s0, n, pos0 = _step_rows(b, seq_lens, query_starts, query_lens)
+        if n <= 0:
+            continue
+        slot = int(state_slots[b])
+        fresh = pos0 <= 0
+        St = torch.zeros(H, Dv, D) if fresh else S[slot].clone()
+        if kind == SCAN_MLSTM:
+            nv = torch.zeros(H, D) if fresh else n_state[slot].clone()
+            mv = torch.zeros(H) if fresh else m_state[slot].clone()
+        for t in range(s0, s0 + n):
+            qt = q[t].float().repeat_interleave(rep, 0) * q_scale   # [H, D]
+            kt = k[t].float().repeat_interleave(rep, 0)
+            vt = v[t].float()                                       # [H, Dv]
+            z = gate[t].float()
+            if kind == SCAN_GLA:
+                a = torch.exp(lsig(z + gb) * gate_param).view(H, D)
+                St = St * a.unsqueeze(1) + vt.unsqueeze(2) * kt.unsqueeze(1)
+                out[t] = torch.einsum("hvd,hd->hv", St, qt)
+            elif kind == SCAN_DELTA:
+                g = torch.exp(-torch.exp(head_rate.float()).view(H, 1)
+                              * torch.nn.functional.softplus(
+                                  (z + gb).view(H, D)))
+                St = St * g.unsqueeze(1)
+                bt = torch.sigmoid(beta[t].float()).view(H, 1)
+                u = bt * (vt - torch.einsum("hvd,hd->hv", St, kt))
+                St = St + u.unsqueeze(2) * kt.unsqueeze(1)
+                out[t] = torch.einsum("hvd,hd->hv", St, qt)
+            else:
+                c = gate_param
+                zb = z + gb
+                ig = c * torch.tanh(zb[:H] / c)
+                fg = lsig(c * torch.tanh(zb[H:] / c))
+                mn = torch.maximum(fg + mv, ig)
+                df = torch.exp(fg + mv - mn).view(H, 1)
+                di = torch.exp(ig - mn).view(H, 1)
+                St = (St * df.unsqueeze(2)
+                      + (di * vt).unsqueeze(2) * kt.unsqueeze(1))
+                nv = nv * df + di * kt
+                mv = mn
+                den = torch.maximum((nv * qt).sum(-1).abs(),
+                                    torch.exp(-mv)) + 1e-6
+                out[t] = torch.einsum("hvd,hd->hv", St, qt) / den.view(H, 1)
+        S[slot] = St
+        if kind == SCAN_MLSTM:
+            n_state[slot] = nv
+            m_state[slot] = mv
+
+
+def head_rmsnorm_gate(out: torch.Tensor, o: torch.Tensor, w: torch.Tensor,
+                      gate: torch.Tensor, eps: float, silu_gate: bool) -> None:
+    """out[t, h*Dv + e] = o[t, h, e] / rms_e(o[t, h]) * w * act(gate):
+    o fp32 [T, H, Dv]; w has Dv entries (shared by the heads) or H*Dv;
+    act = silu or sigmoid of gate [T, H*Dv]."""
+    T, H, Dv = o.shape
+    r = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+    wf = w.float()
+    r = r * (wf.view(1, 1, Dv) if wf.numel() == Dv else wf.view(1, H, Dv))
+    g = gate.float().reshape(T, H, Dv)
+    a = g * torch.sigmoid(g) if silu_gate else torch.sigmoid(g)
+    out.copy_((r * a).reshape(T, H * Dv).to(out.dtype))
+
+
+def grouped_softmax_route(weight: torch.Tensor, logits: torch.Tensor,
+                          correction, top: int, n_groups: int,
+                          keep_groups: int, scale: float) -> None:
+    """Dense routing weights [T, E] (0 = not chosen), fp32 throughout.
+    s = softmax(logits); choice score c = s + correction; experts form
+    n_groups equal consecutive groups, a group scores max(c) over its
+    members and only the keep_groups best groups stay eligible; the `top`
+    eligible experts with the largest c are chosen and weigh
+    s / (sum of chosen s + 1e-20) * scale."""
+    T, E = logits.shape
+    s = torch.softmax(logits.float(), dim=-1)
+    c = s if correction is None else s + correction.float()
+    if n_groups > 1 and keep_groups < n_groups:
+        gs = c.view(T, n_groups, E // n_groups).max(-1).values
+        keep = torch.zeros(T, n_groups, dtype=torch.bool)
+        keep.scatter_(1, gs.topk(keep_groups, dim=-1).indices, True)
+        ok = keep.unsqueeze(-1).expand(T, n_groups, E // n_groups)
+        c = c.masked_fill(~ok.reshape(T, E), float("-inf"))
+    idx = c.topk(top, dim=-1).indices
+    ws = s.gather(1, idx)
+    ws = ws / (ws.sum(-1, keepdim=True) + 1e-20) * scale
+    weight.zero_()
+    weight.scatter_(1, idx, ws)
+
+
+def routed_clamped_glu(out: torch.Tensor, gu: torch.Tensor,
+                       weight: torch.Tensor, n_experts: int, limit: float,
+                       slope: float) -> None:
+    """Stacked-expert activation with the routing weight on the OUTPUT
+    side: gu [T, E*2F] (expert e: gate | up), weight [T, >= E] (columns
+    past n_experts belong to weightless experts and are ignored);
+    g = min(gate, limit), u = clamp(up, -limit, limit);
+    out[t, e, :] = weight[t, e] * g * sigmoid(slope * g) * (u + 1), and 0
+    where the weight is 0."""
+    T = gu.size(0)
+    E = n_experts
+    F_ = gu.size(1) // (2 * E)
+    g3 = gu.view(T, E, 2 * F_).float()
+    g = g3[..., :F_].clamp(max=limit)
+    u = g3[..., F_:].clamp(-limit, limit)
+    w = weight[:, :E].float().unsqueeze(-1)
+    y = g * torch.sigmoid(slope * g) * (u + 1.0) * w
+    y = torch.where(w == 0, torch.zeros_like(y), y)
+    out.copy_(y.view(T, E * F_).to(out.dtype))
