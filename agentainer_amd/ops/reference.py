@@ -563,7 +563,8 @@ def short_conv_state(out: torch.Tensor, u: torch.Tensor, w: torch.Tensor,
         if n <= 0:
             continue
         slot = int(state_slots[b])
-        hist = tail[slot].float() if pos0 > 0 else torch.zeros_like(tail[slot])
+        hist = tail[slot].float().clone()
+        hist[:max(0, taps - 1 - max(pos0, 0))] = 0      # before position 0
         full = torch.cat([hist, u[s0:s0 + n].float()], dim=0)
         y = torch.zeros(n, u.size(1))
         for j in range(taps):
