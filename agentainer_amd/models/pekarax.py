@@ -142,7 +142,7 @@ class PekaraxConfig:
         for l in self.layers:
             d: Dict[str, tuple] = {}
             a, m = l.attn, l.memory
-            if a is not None and a.conv_taps > 1:
+            if a is not None and a.conv_taps > 0:
                 ch = a.heads * a.dim + a.kv_heads * (a.dim + a.vdim)
                 d["attn_conv"] = (a.conv_taps - 1, ch)
             if m is not None:
@@ -150,7 +150,7 @@ class PekaraxConfig:
                 if m.kind == ops.SCAN_MLSTM:
                     d["n"] = (m.heads, m.dim)
                     d["m"] = (m.heads,)
-                if m.conv_taps > 1:
+                if m.conv_taps > 0:
                     d["conv"] = (m.conv_taps - 1,
                                  2 * m.qk_heads * m.dim + m.heads * m.vdim)
             out.append(d)
