@@ -86,7 +86,7 @@ def _parser():
                    help="--arch-compare: which size points to run "
                         "(default: all points of the design)")
     p.add_argument("--arch-design", default="lelitar",
-                   choices=["lelitar", "volalorn"],
+                   choices=["lelitar", "volalorn", "pekarax"],
                    help="--arch-compare: which design to measure")
     return p
 
@@ -181,6 +181,60 @@ def _volalorn_points():
     }
 
 
+def _pekarax_points():
+    """Pekarax size points beside Mixtral stacks of equal width, attention
+    head counts, expert count, expert size and top-k: four layers
+    (channel-delta, parallel attention + mLSTM, gated linear attention,
+    channel-delta), every one followed by the routed experts (two identity
+    experts on top of the weighted ones, two groups of which one is
+    kept)."""
+    from agentainer_amd import ops
+    from agentainer_amd.models.mixtral import MixtralConfig
+    from agentainer_amd.models.pekarax import (GroupedExpertsConfig,
+                                               MatrixMemoryConfig,
+                                               PekaraxConfig,
+                                               PekaraxLayerConfig)
+    from agentainer_amd.models.volalorn import MaskedAttentionConfig
+
+    def pek(name, width, heads, kv, ff, experts, top):
+        ex = GroupedExpertsConfig(experts=experts, identity=2, top=top, ff=ff,
+                                  limit=7.0, groups=2, keep_groups=1,
+                                  scale=2.5)
+        hv = width // 128
+        delta = MatrixMemoryConfig(ops.SCAN_DELTA, hv, hv // 2, 128, 128,
+                                   conv_taps=4, decay_rank=64, gate_rank=64)
+        gla = MatrixMemoryConfig(ops.SCAN_GLA, hv // 2, hv // 2, 128, 256,
+                                 decay_rank=64, tau=16.0)
+        mlstm = MatrixMemoryConfig(ops.SCAN_MLSTM, hv // 2, hv // 2, 128, 256,
+                                   gate_cap=15.0)
+        attn = MaskedAttentionConfig(
+            heads=heads, kv_heads=kv, dim=128, vdim=128, scale=0.09,
+            mask_kind=ops.MASK_CAUSAL, mask_size=0, rot_dims=64,
+            rot_base=500000.0, conv_taps=3)
+        layers = [PekaraxLayerConfig("channel_delta", memory=delta, mlp=ex),
+                  PekaraxLayerConfig("parallel", attn=attn, memory=mlstm,
+                                     attn_scale=0.8, memory_scale=0.9, mlp=ex),
+                  PekaraxLayerConfig("gla", memory=gla, mlp=ex),
+                  PekaraxLayerConfig("channel_delta", memory=delta, mlp=ex)]
+        return PekaraxConfig(name=name, vocab_size=32000, hidden_size=width,
+                             layers=layers, norm_eps=1e-5, postln_alpha=2.5)
+
+    return {
+        "s": ("w2048-8x4096-top2", pek("pekarax-s", 2048, 16, 4, 4096, 8, 2),
+              MixtralConfig(name="mixtral-s", vocab_size=32000,
+                            hidden_size=2048, n_layers=4, n_heads=16,
+                            n_kv_heads=4, intermediate_size=4096,
+                            n_experts=8, top_k=2, tie_embeddings=False),
+              "mixtral"),
+        "l": ("w4096-8x7168-top2", pek("pekarax-l", 4096, 32, 8, 7168, 8, 2),
+              MixtralConfig(name="mixtral-l", vocab_size=32000,
+                            hidden_size=4096, n_layers=4, n_heads=32,
+                            n_kv_heads=8, intermediate_size=7168,
+                            n_experts=8, top_k=2, tie_embeddings=False),
+              "mixtral"),
+    }
+
+
 def run_arch_compare(args):
     """Prefill (8 x 1024-token prompts per step) and decode (64 sequences at
     1024 tokens of context, captured graph) throughput, through the
@@ -188,6 +242,7 @@ def run_arch_compare(args):
     from agentainer_amd.engine.llm import ModelInstance
     from agentainer_amd.models.lelitar import LelitarForCausalLM
     from agentainer_amd.models.mixtral import MixtralForCausalLM
+    from agentainer_amd.models.pekarax import PekaraxForCausalLM
     from agentainer_amd.models.volalorn import VolalornForCausalLM
 
     dev = "cuda" if torch.cuda.is_available() else "cpu"
@@ -247,9 +302,11 @@ def run_arch_compare(args):
                 "decode_tok_s": round(n_dec / dc * 1e3)}
 
     design = args.arch_design
-    pts = _volalorn_points() if design == "volalorn" else _arch_points()
-    ours_cls = (VolalornForCausalLM if design == "volalorn"
-                else LelitarForCausalLM)
+    pts = {"volalorn": _volalorn_points, "pekarax": _pekarax_points,
+           "lelitar": _arch_points}[design]()
+    ours_cls = {"volalorn": VolalornForCausalLM,
+                "pekarax": PekaraxForCausalLM,
+                "lelitar": LelitarForCausalLM}[design]
     for key in (args.arch_sizes or ",".join(pts)).split(","):
         label, lcfg, rcfg, kind = pts[key.strip()]
         if small:  # CPU dry run: shrink to something that finishes
