@@ -747,6 +747,11 @@ def short_conv_state(out, u, w, tail, state_slots, seq_lens, query_starts,
     return out
 
 
+# lanes that share one value column in the recurrence kernel; 0 = sized per
+# launch (A/B runs)
+SCAN_LANES = int(os.environ.get("AGENTAINER_SCAN_LANES", "0"))
+
+
 def matrix_memory_scan(kind: int, out, q, k, v, gate, gate_bias, head_rate,
                        beta, q_scale: float, gate_param: float, S, n_state,
                        m_state, state_slots, seq_lens, query_starts,
@@ -757,7 +762,7 @@ def matrix_memory_scan(kind: int, out, q, k, v, gate, gate_bias, head_rate,
                                head_rate, beta, float(q_scale),
                                float(gate_param), S, n_state, m_state,
                                state_slots, seq_lens, query_starts,
-                               query_lens)
+                               query_lens, int(SCAN_LANES))
     else:
         reference.matrix_memory_scan(kind, out, q, k, v, gate, gate_bias,
                                      head_rate, beta, q_scale, gate_param, S,

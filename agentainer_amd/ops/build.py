@@ -55,6 +55,9 @@ RECURRENT_SOURCES = [
     "postln_norm.hip",
     "short_conv.hip",
     "matrix_memory.hip",
+    "matrix_memory_gla.hip",
+    "matrix_memory_delta.hip",
+    "matrix_memory_mlstm.hip",
     "grouped_route.hip",
 ]
 
@@ -104,6 +107,7 @@ def needs_build(target: str = "core") -> bool:
     srcs = [os.path.join(CSRC, s) for s in SOURCES]
     srcs.append(os.path.join(CSRC, "common.h"))
     srcs.append(os.path.join(CSRC, "latent_common.h"))
+    srcs.append(os.path.join(CSRC, "matrix_memory_kernel.h"))
     srcs.append(os.path.abspath(__file__))
     return _newest(srcs) > os.path.getmtime(OUT)
 
@@ -144,7 +148,8 @@ def build(verbose: bool = True, force: bool = False,
         if (os.path.exists(obj)
                 and os.path.getmtime(obj) > _newest(
                     [src_path, os.path.join(CSRC, "common.h"),
-                     os.path.join(CSRC, "latent_common.h")])
+                     os.path.join(CSRC, "latent_common.h"),
+                     os.path.join(CSRC, "matrix_memory_kernel.h")])
                 and not force):
             continue
         san = (["-fsanitize=address", "-shared-libsan"]

@@ -20,7 +20,7 @@ void matrix_memory_scan(long kind, torch::Tensor out, torch::Tensor q,
                         double q_scale, double gate_param, torch::Tensor S,
                         OptT n_state, OptT m_state, torch::Tensor state_slots,
                         torch::Tensor seq_lens, OptT query_starts,
-                        OptT query_lens);
+                        OptT query_lens, long lanes);
 void head_rmsnorm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor w,
                        torch::Tensor gate, double eps, bool silu_gate);
 void grouped_softmax_route(torch::Tensor weight, torch::Tensor logits,

@@ -214,3 +214,51 @@ def test_routed_clamped_glu(dtype, F_):
     tol = 1e-5 if dtype == torch.float32 else 2e-2
     torch.testing.assert_close(outg.cpu().float(), outr.float(), rtol=tol,
                                atol=tol)
+
+
+@pytest.mark.parametrize("kind", [ops.SCAN_GLA, ops.SCAN_DELTA,
+                                  ops.SCAN_MLSTM])
+@pytest.mark.parametrize("D,Dv,H,B", [(32, 256, 16, 64), (64, 128, 16, 64),
+                                      (128, 128, 16, 32), (256, 128, 8, 32)])
+def test_matrix_memory_scan_many_columns(kind, D, Dv, H, B):
+    """Launches with many (sequence, head, column) triples take the
+    variant with the fewest lanes per column; a decode step and a step of
+    short portions."""
+    _need()
+    g = torch.Generator().manual_seed(D)
+    for decode in (True, False):
+        new = [1] * B if decode else [2] * B
+        before = [(3 * i) % 5 for i in range(B)]
+        seq, qs, ql = _step(new, before, decode)
+        T = sum(new)
+        slots = torch.randperm(B + 3, generator=g)[:B]
+        q = torch.randn(T, H, D, generator=g)
+        k = torch.randn(T, H, D, generator=g) / D ** 0.5
+        v = torch.randn(T, H, Dv, generator=g)
+        if kind == ops.SCAN_MLSTM:
+            gate = torch.randn(T, 2 * H, generator=g) * 3
+            bias = torch.randn(2 * H, generator=g)
+        else:
+            gate = torch.randn(T, H * D, generator=g) * 2
+            bias = torch.randn(H * D, generator=g)
+        rate = torch.randn(H, generator=g) * 0.5
+        beta = torch.randn(T, H, generator=g)
+        S = torch.randn(B + 3, H, Dv, D, generator=g)
+        n_st = torch.randn(B + 3, H, D, generator=g)
+        m_st = torch.randn(B + 3, H, generator=g)
+        param = {ops.SCAN_GLA: 0.25, ops.SCAN_DELTA: 0.0,
+                 ops.SCAN_MLSTM: 9.0}[kind]
+        Sr, nr, mr = S.clone(), n_st.clone(), m_st.clone()
+        outr = torch.zeros(T, H, Dv)
+        ref.matrix_memory_scan(kind, outr, q, k, v, gate, bias, rate, beta,
+                               0.5, param, Sr, nr, mr, slots, seq, qs, ql)
+        Sg, ng, mg = S.to(DEV), n_st.to(DEV), m_st.to(DEV)
+        outg = torch.zeros(T, H, Dv, device=DEV)
+        ops.matrix_memory_scan(kind, outg, q.to(DEV), k.to(DEV), v.to(DEV),
+                               gate.to(DEV), bias.to(DEV), rate.to(DEV),
+                               beta.to(DEV), 0.5, param, Sg, ng, mg,
+                               slots.to(DEV), seq.to(DEV), _dev(qs), _dev(ql))
+        torch.testing.assert_close(outg.cpu(), outr, rtol=2e-4, atol=2e-4)
+        torch.testing.assert_close(Sg.cpu(), Sr, rtol=2e-4, atol=2e-4)
+        if kind == ops.SCAN_MLSTM:
+            torch.testing.assert_close(ng.cpu(), nr, rtol=2e-4, atol=2e-4)
