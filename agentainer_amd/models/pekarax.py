@@ -332,7 +332,7 @@ class MatrixMemoryMixer(torch.nn.Module):
             self.g2 = _param(H * Dv, mc.gate_rank, dtype=f32)
             self.head_rate = _param(H, dtype=f32)
         self.conv_channels = self.q_sz + self.k_sz + self.v_sz
-        self.w_conv = (_param(self.conv_channels, mc.conv_taps, dtype=f32)
+        self.w_conv = (_param(mc.conv_taps, self.conv_channels, dtype=f32)
                        if mc.conv_taps > 0 else None)
         self.w_o = _param(width, H * Dv, dtype=dtype)
 
@@ -363,8 +363,9 @@ class MatrixMemoryMixer(torch.nn.Module):
             self.gate_bias.copy_(torch.cat([f("i.b"), f("f.b")], dim=0))
         self.norm_w.copy_(f("norm"))
         if mc.conv_taps > 0:
+            # checkpoint [channels, taps] -> tap-major [taps, channels]
             self.w_conv.copy_(torch.cat([f("q.conv"), f("k.conv"),
-                                         f("v.conv")], dim=0))
+                                         f("v.conv")], dim=0).t())
         self.w_o.copy_(get("o"))
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, state: dict,

@@ -212,7 +212,7 @@ class MaskedAttention(torch.nn.Module):
         self.key_bias = _param(H, dtype=f32) if mc.key_bias else None
         self.w_o = _param(width, H * mc.vdim, dtype=dtype)
         self.conv_channels = self.q_sz + self.k_sz + self.v_sz
-        self.w_conv = (_param(self.conv_channels, mc.conv_taps, dtype=f32)
+        self.w_conv = (_param(mc.conv_taps, self.conv_channels, dtype=f32)
                        if mc.conv_taps > 0 else None)
         freqs, self.rot_amp = ops.rotary_frequencies(
             mc.rot_dims, mc.rot_base, mc.rot_scaling)
@@ -241,8 +241,10 @@ class MaskedAttention(torch.nn.Module):
             self.key_bias.copy_(get("pb").float())
         self.w_o.copy_(get("o"))
         if mc.conv_taps > 0:
+            # checkpoint [channels, taps] -> tap-major [taps, channels]
             self.w_conv.copy_(torch.cat(
-                [get("q.conv"), get("k.conv"), get("v.conv")], dim=0).float())
+                [get("q.conv"), get("k.conv"), get("v.conv")],
+                dim=0).float().t())
 
     def rotary_key(self):
         """Layers with equal keys share one cos/sin table per step."""

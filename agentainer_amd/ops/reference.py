@@ -550,13 +550,14 @@ def short_conv_state(out: torch.Tensor, u: torch.Tensor, w: torch.Tensor,
     """Depthwise causal convolution over time with the last taps-1 inputs
     of every sequence kept in tail [slots, taps-1, C] (fp32).
 
-    y[t, c] = sum_j w[c, j] * u[t - taps + 1 + j, c]; inputs before this
+    y[t, c] = sum_j w[j, c] * u[t - taps + 1 + j, c] (w is tap-major,
+    [taps, C]); inputs before this
     step's rows come from the tail, inputs before position 0 are zero (a
     sequence whose first row sits at position 0 ignores its tail). Then
     optionally silu, and for the first norm_channels channels, cut into
     heads of head_dim, y / sqrt(sum(y^2) + l2_eps); the first lead_channels
     of those are multiplied by lead_scale. The tail is rewritten."""
-    taps = w.size(1)
+    taps = w.size(0)
     wf = w.float()
     for b in range(seq_lens.numel()):
         s0, n, pos0 = _step_rows(b, seq_lens, query_starts, query_lens)
@@ -568,7 +569,7 @@ def short_conv_state(out: torch.Tensor, u: torch.Tensor, w: torch.Tensor,
         full = torch.cat([hist, u[s0:s0 + n].float()], dim=0)
         y = torch.zeros(n, u.size(1))
         for j in range(taps):
-            y = y + wf[:, j] * full[j:j + n]
+            y = y + wf[j] * full[j:j + n]
         if taps > 1:
             tail[slot] = full[-(taps - 1):]
         if silu:

@@ -72,17 +72,20 @@ def test_postln_rmsnorm_residual(dtype, W):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("taps", [1, 2, 4])
 @pytest.mark.parametrize("decode", [False, True])
-def test_short_conv_state(dtype, taps, decode):
+@pytest.mark.parametrize("D,extra", [(24, 100), (25, 7), (128, 256), (64, 40)])
+def test_short_conv_state(dtype, taps, decode, D, extra):
+    """Sizes that take the four-channels-per-lane kernel (8, 16, 32 lanes
+    per head) and sizes that do not."""
     _need()
     g = torch.Generator().manual_seed(taps)
-    heads, D = 3, 24
-    C = 2 * heads * D + 100
+    heads = 3
+    C = 2 * heads * D + extra
     new = [1, 1, 1] if decode else [5, 1, 2, 9]
     before = [0, 3, 7] if decode else [0, 4, 1, 0]
     seq, qs, ql = _step(new, before, decode)
     T, B = sum(new), len(new)
     u = torch.randn(T, C + 8, generator=g).to(dtype)[:, :C]
-    w = torch.randn(C, taps, generator=g)
+    w = torch.randn(taps, C, generator=g)
     tail = torch.randn(6, taps - 1, C, generator=g)
     slots = torch.tensor([4, 0, 2, 5][:B], dtype=torch.long)
     for out_dt, kw in ((torch.float32, dict(silu=True,

@@ -96,7 +96,7 @@ def test_short_conv_tail_over_cuts(device, taps, sizes):
         k += 1
         md = step_md(device, [n], [at], [1], decode=(n == 1 and at > 0))
         ops.short_conv_state(out[at:at + n], u[at:at + n].to(device),
-                             w.to(device), tail, md.state_slots, md.seq_lens,
+                             w.t().contiguous().to(device), tail, md.state_slots, md.seq_lens,
                              md.query_starts, md.query_lens)
         at += n
     assert rel(out, want) < 1e-5
