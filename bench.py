@@ -199,12 +199,12 @@ def _pekarax_points():
     def pek(name, width, heads, kv, ff, experts, top):
         ex = GroupedExpertsConfig(experts=experts, identity=2, top=top, ff=ff,
                                   limit=7.0, groups=2, keep_groups=1,
-                                  scale=2.5)
+                                  scale=2.0)
         hv = width // 128
         delta = MatrixMemoryConfig(ops.SCAN_DELTA, hv, hv // 2, 128, 128,
                                    conv_taps=4, decay_rank=64, gate_rank=64)
         gla = MatrixMemoryConfig(ops.SCAN_GLA, hv // 2, hv // 2, 128, 256,
-                                 decay_rank=64, tau=16.0)
+                                 decay_rank=64, tau=8.0)
         mlstm = MatrixMemoryConfig(ops.SCAN_MLSTM, hv // 2, hv // 2, 128, 256,
                                    gate_cap=15.0)
         attn = MaskedAttentionConfig(
@@ -217,7 +217,7 @@ def _pekarax_points():
                   PekaraxLayerConfig("gla", memory=gla, mlp=ex),
                   PekaraxLayerConfig("channel_delta", memory=delta, mlp=ex)]
         return PekaraxConfig(name=name, vocab_size=32000, hidden_size=width,
-                             layers=layers, norm_eps=1e-5, postln_alpha=2.5)
+                             layers=layers, norm_eps=1e-5, postln_alpha=2.0)
 
     return {
         "s": ("w2048-8x4096-top2", pek("pekarax-s", 2048, 16, 4, 4096, 8, 2),

@@ -239,7 +239,7 @@ def delta_layer(heads=4, kv_heads=2, dim=8, vdim=6, conv=4, rank=4, grank=5):
 
 
 def parallel_layer(heads=4, kv_heads=2, dim=8, vdim=6, conv=3, rot_dims=4,
-                   base=100.0, scale=0.7, left_scale=0.8, right_scale=1.2,
+                   base=100.0, scale=0.7, left_scale=0.75, right_scale=1.2,
                    m_heads=2, m_dim=8, m_vdim=10, cap=8.0):
     return {"type": "parallel", "mixer": {
         "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim,

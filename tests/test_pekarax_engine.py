@@ -335,10 +335,10 @@ def test_named_random_init_model_is_registered(tmp_path):
                     grank=8),
       O.parallel_layer(heads=8, kv_heads=2, dim=64, vdim=64, conv=3,
                        rot_dims=32, scale=0.1, m_heads=2, m_dim=32,
-                       m_vdim=64, cap=12.0),
-      O.gla_layer(heads=2, dim=128, vdim=64, tau=16.0, rank=8)],
+                       m_vdim=64, cap=11.0),
+      O.gla_layer(heads=2, dim=128, vdim=64, tau=12.0, rank=8)],
      dict(width=128, mlp=O.moe(experts=8, identity=2, top=3, ff=64,
-                               limit=2.0, groups=2, keep=1))),
+                               limit=1.8, groups=2, keep=1))),
     # head sizes the attention tile kernel does not take -> row kernel
     ([O.parallel_layer(heads=3, kv_heads=1, dim=24, vdim=20, conv=2,
                        rot_dims=8, m_heads=3, m_dim=40, m_vdim=12),

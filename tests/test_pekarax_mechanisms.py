@@ -293,7 +293,7 @@ def test_group_limited_choice_with_negative_scores(device):
     corr = -1.0 - torch.rand(E, generator=g)
     wt = torch.empty(T, E, device=device)
     ops.grouped_softmax_route(wt, logits.to(device), corr.to(device), 3, 4, 2,
-                              2.5)
+                              1.75)
     wt = wt.cpu()
     s = torch.softmax(logits.double(), -1)
     c = s + corr.double()
@@ -303,9 +303,9 @@ def test_group_limited_choice_with_negative_scores(device):
                       key=lambda e: -float(c[t, e]))[:3]
         chosen = sorted(int(e) for e in wt[t].nonzero().flatten())
         assert chosen == sorted(cand), t
-        want = s[t, cand] / s[t, cand].sum() * 2.5
+        want = s[t, cand] / s[t, cand].sum() * 1.75
         assert rel(wt[t, cand], want) < 1e-5
-    assert rel(wt.sum(-1), torch.full((T,), 2.5)) < 1e-5
+    assert rel(wt.sum(-1), torch.full((T,), 1.75)) < 1e-5
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -343,7 +343,7 @@ def test_config_reader_takes_ranks_from_tensor_shapes(tmp_path):
     assert pc.layers[0].memory.decay_rank == 3
     assert pc.layers[0].memory.gate_rank == 7
     assert pc.layers[1].memory.decay_rank == 5 and pc.layers[1].mlp is None
-    assert pc.layers[2].attn.conv_taps == 3 and pc.layers[2].attn_scale == 0.8
+    assert pc.layers[2].attn.conv_taps == 3 and pc.layers[2].attn_scale == 0.75
     assert pc.layers[2].memory.kind == ops.SCAN_MLSTM
     shapes = pc.state_shapes()
     assert shapes[0]["S"] == (4, 6, 8) and shapes[0]["conv"] == (3, 56)
