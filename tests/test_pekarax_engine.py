@@ -350,6 +350,11 @@ def test_bf16_serving_path_close_to_oracle(tmp_path, layers, kw):
     step after step."""
     cfg = O.make_config(layers, vocab=300, **kw)
     w = O.random_weights(cfg, seed=11)
+    for k in w:
+        # peaky routers: near-ties (which bf16 rounding may flip) then sit
+        # among experts of small weight
+        if k.endswith("mlp.router"):
+            w[k] = (w[k] * 4).bfloat16().float()
     eng, inst, _ = make_instance(tmp_path, cfg, w, "cuda", dtype="bfloat16",
                                  page=16, pool_tokens=512)
     reqs = {"a": tokens_for(cfg, 120, 1), "b": tokens_for(cfg, 75, 2)}
