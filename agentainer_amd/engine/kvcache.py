@@ -148,21 +148,29 @@ class HybridStateLayout:
     """Layers that cache per-token K/V pages, per-SEQUENCE state, or both.
 
     kv_shapes[l] is (kv_heads, key_dim, value_dim) — pools as in
-    HeadKVLayout — or None for a layer without attention. state_shapes[l]
-    maps a name to the shape of one sequence's fp32 state tensor of that
-    layer (a recurrent memory, the tail of a short convolution); the
-    manager allocates each as [slots, *shape], indexed by the sequence
-    slot, so a sequence's state is addressed on the device by the same
-    number as its page-table row. The kernels treat a sequence that
-    starts at position 0 as having zero state, so a slot needs no
-    clearing when it is handed to the next sequence."""
+    HeadKVLayout —, a 1-tuple (rank,) — one latent pool [P, PS, rank] as
+    in LatentLayout, handed out as (pool, None) —, or None for a layer
+    that caches nothing per token (no attention, or attention that reads
+    another layer's pools). state_shapes[l]
+    maps a name to the shape of one sequence's state tensor of that
+    layer (a recurrent memory, the tail of a short convolution, the last
+    token id); the manager allocates each as [slots, *shape], indexed by
+    the sequence slot, so a sequence's state is addressed on the device by
+    the same number as its page-table row. States are fp32 unless
+    state_dtypes[l] names another dtype (integers below 2^24 survive the
+    fp32 checkpoint image). The kernels treat a sequence that starts at
+    position 0 as having zero state, so a slot needs no clearing when it
+    is handed to the next sequence."""
 
-    def __init__(self, kv_shapes, state_shapes):
+    def __init__(self, kv_shapes, state_shapes, state_dtypes=None):
         self.kv_shapes = [None if s is None else tuple(int(v) for v in s)
                           for s in kv_shapes]
         self.state_shapes = [{k: tuple(int(x) for x in v)
                               for k, v in d.items()} for d in state_shapes]
+        self.state_dtypes = (state_dtypes if state_dtypes is not None
+                             else [{} for _ in self.state_shapes])
         assert len(self.kv_shapes) == len(self.state_shapes)
+        assert len(self.state_dtypes) == len(self.state_shapes)
         self.n_layers = len(self.kv_shapes)
 
     def alloc(self, n_pages, page_size, device, dtype):
@@ -170,6 +178,9 @@ class HybridStateLayout:
         for s in self.kv_shapes:
             if s is None:
                 out.append((None, None))
+            elif len(s) == 1:
+                out.append((torch.zeros(n_pages, page_size, s[0], dtype=dtype,
+                                        device=device), None))
             else:
                 g, d, dv = s
                 out.append((torch.zeros(n_pages, g, page_size, d, dtype=dtype,
@@ -179,13 +190,14 @@ class HybridStateLayout:
         return out
 
     def alloc_state(self, n_slots, device):
-        return [{k: torch.zeros(n_slots, *shape, dtype=torch.float32,
+        return [{k: torch.zeros(n_slots, *shape,
+                                dtype=dt.get(k, torch.float32),
                                 device=device) for k, shape in d.items()}
-                for d in self.state_shapes]
+                for d, dt in zip(self.state_shapes, self.state_dtypes)]
 
     def page_elems(self, page_size: int) -> int:
-        return max([g * (d + dv) for g, d, dv in
-                    (s for s in self.kv_shapes if s is not None)] + [1]
+        return max([s[0] if len(s) == 1 else s[0] * (s[1] + s[2])
+                    for s in self.kv_shapes if s is not None] + [1]
                    ) * page_size
 
     def state_elems(self) -> int:
@@ -212,11 +224,19 @@ class HybridStateLayout:
         return tot
 
     def gather(self, entry, staging, page_ids):
-        if entry[0] is not None:
+        if entry[0] is None:
+            return
+        if entry[1] is None:
+            LatentLayout.gather(self, entry, staging, page_ids)
+        else:
             HeadKVLayout.gather(self, entry, staging, page_ids)
 
     def scatter(self, entry, staging, page_ids):
-        if entry[0] is not None:
+        if entry[0] is None:
+            return
+        if entry[1] is None:
+            LatentLayout.scatter(self, entry, staging, page_ids)
+        else:
             HeadKVLayout.scatter(self, entry, staging, page_ids)
 
     def gather_state(self, state, slot: int, row: torch.Tensor) -> None:
@@ -224,7 +244,7 @@ class HybridStateLayout:
         off = 0
         for k in sorted(state):
             t = state[k][slot].reshape(-1)
-            row[off:off + t.numel()] = t
+            row[off:off + t.numel()] = t.to(row.dtype)
             off += t.numel()
 
     def scatter_state(self, state, slot: int, row: torch.Tensor) -> None:
@@ -232,7 +252,7 @@ class HybridStateLayout:
         for k in sorted(state):
             n = state[k][slot].numel()
             state[k][slot] = row[off:off + n].view(state[k].shape[1:]).to(
-                state[k].device)
+                device=state[k].device, dtype=state[k].dtype)
             off += n
 
 

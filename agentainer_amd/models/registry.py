@@ -21,6 +21,10 @@ FAMILIES: Dict[str, Tuple[str, str, str, str]] = {
     # convolved attention reuses the masked-attention kernels
     "Pekarax": ("agentainer_amd.models.pekarax", "PEKARAX_CONFIGS",
                 "make_pekarax_instance", "masked+recurrent"),
+    # window attention on the masked-attention kernels, latent attention
+    # on the latent ones, convolution tails from the recurrent module
+    "Sipelorn": ("agentainer_amd.models.sipelorn", "SIPELORN_CONFIGS",
+                 "make_sipelorn_instance", "gated+masked+latent+recurrent"),
 }
 
 

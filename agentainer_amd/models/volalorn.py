@@ -89,6 +89,14 @@ class MaskedAttentionConfig:
     #                           on the projected q, k, v (before norm and
     #                           rotary); its last taps-1 inputs are
     #                           per-sequence state
+    plain_qk: bool = False    # q and k enter the scores as projected (and
+    #                           convolved): no rotary, no norm
+    dist_bias: bool = False   # per head (r1, r2): r1 ln(1 + r2 (p - j)) is
+    #                           taken off the score of key j at query p
+    elem_gate: bool = False   # sigmoid gate per OUTPUT COORDINATE, read
+    #                           from the mixer input
+    kv_from: Optional[int] = None   # this layer has no k/v projections: it
+    #                           attends the pools of that (earlier) layer
 
 
 @dataclass
@@ -190,26 +198,42 @@ def _param(*shape, dtype):
                               requires_grad=False)
 
 
+def _align(n: int) -> int:
+    return -(-n // PROJ_ALIGN) * PROJ_ALIGN
+
+
 class MaskedAttention(torch.nn.Module):
     """Grouped-query attention with a configurable mask, weighting, q/k
     normalization order and output gate (see MaskedAttentionConfig)."""
 
     def __init__(self, width: int, mc: MaskedAttentionConfig, eps: float,
-                 dtype):
+                 dtype, extra_rows: int = 0):
+        """extra_rows: that many more rows ride in the input GEMM (a
+        projection of the same input that belongs to the caller, e.g. a
+        residual gate); forward then returns (output, their columns)."""
         super().__init__()
         self.mc = mc
         self.eps = eps
         H, G = mc.heads, mc.kv_heads
-        self.q_sz, self.k_sz, self.v_sz = H * mc.dim, G * mc.dim, G * mc.vdim
-        n = self.q_sz + self.k_sz + self.v_sz + (H if mc.head_gate else 0)
-        self.n_in = -(-n // PROJ_ALIGN) * PROJ_ALIGN
-        # one GEMM from the mixer input: [q | k | v | head-gate logits]
+        own_kv = mc.kv_from is None
+        self.q_sz = H * mc.dim
+        self.k_sz = G * mc.dim if own_kv else 0
+        self.v_sz = G * mc.vdim if own_kv else 0
+        self.gate_sz = (H if mc.head_gate else
+                        H * mc.vdim if mc.elem_gate else 0)
+        # segment starts stay 16-byte aligned for the kernels' vector loads
+        self.gate_off = _align(self.q_sz + self.k_sz + self.v_sz)
+        self.extra_rows = extra_rows
+        self.extra_off = _align(self.gate_off + self.gate_sz)
+        self.n_in = _align(self.extra_off + extra_rows)
+        # one GEMM from the mixer input: [q | k | v | gate logits | extra]
         self.w_in = _param(self.n_in, width, dtype=dtype)
         self.b_in = _param(self.n_in, dtype=dtype) if mc.qkv_bias else None
         f32 = torch.float32
         self.q_norm = _param(mc.dim, dtype=f32) if mc.norm_first else None
         self.k_norm = _param(mc.dim, dtype=f32) if mc.norm_first else None
         self.key_bias = _param(H, dtype=f32) if mc.key_bias else None
+        self.dist_bias = _param(H, 2, dtype=f32) if mc.dist_bias else None
         self.w_o = _param(width, H * mc.vdim, dtype=dtype)
         self.conv_channels = self.q_sz + self.k_sz + self.v_sz
         self.w_conv = (_param(mc.conv_taps, self.conv_channels, dtype=f32)
@@ -219,32 +243,43 @@ class MaskedAttention(torch.nn.Module):
         self.register_buffer("rot_freqs", freqs, persistent=False)
 
     @torch.no_grad()
-    def load(self, get):
+    def load(self, get, extra=None):
+        """extra: weight rows [extra_rows, width] of the caller's
+        projection."""
         mc = self.mc
+        own_kv = mc.kv_from is None
         q0, k0, v0 = 0, self.q_sz, self.q_sz + self.k_sz
-        g0 = v0 + self.v_sz
+        g0 = self.gate_off
         self.w_in.zero_()
         self.w_in[q0:k0].copy_(get("q"))
-        self.w_in[k0:v0].copy_(get("k"))
-        self.w_in[v0:g0].copy_(get("v"))
-        if mc.head_gate:
-            self.w_in[g0:g0 + mc.heads].copy_(get("g"))
+        if own_kv:
+            self.w_in[k0:v0].copy_(get("k"))
+            self.w_in[v0:v0 + self.v_sz].copy_(get("v"))
+        if self.gate_sz:
+            self.w_in[g0:g0 + self.gate_sz].copy_(get("g"))
+        if extra is not None:
+            self.w_in[self.extra_off:self.extra_off + self.extra_rows].copy_(
+                extra)
         if mc.qkv_bias:
             self.b_in.zero_()
             self.b_in[q0:k0].copy_(get("q.b"))
-            self.b_in[k0:v0].copy_(get("k.b"))
-            self.b_in[v0:g0].copy_(get("v.b"))
+            if own_kv:
+                self.b_in[k0:v0].copy_(get("k.b"))
+                self.b_in[v0:v0 + self.v_sz].copy_(get("v.b"))
         if mc.norm_first:
             self.q_norm.copy_(get("q.norm").float())
             self.k_norm.copy_(get("k.norm").float())
         if mc.key_bias:
             self.key_bias.copy_(get("pb").float())
+        if mc.dist_bias:
+            self.dist_bias.copy_(torch.stack(
+                [get("r1").float(), get("r2").float()], dim=1))
         self.w_o.copy_(get("o"))
         if mc.conv_taps > 0:
             # checkpoint [channels, taps] -> tap-major [taps, channels]
-            self.w_conv.copy_(torch.cat(
-                [get("q.conv"), get("k.conv"), get("v.conv")],
-                dim=0).float().t())
+            names = ["q.conv"] + (["k.conv", "v.conv"] if own_kv else [])
+            self.w_conv.copy_(torch.cat([get(n) for n in names],
+                                        dim=0).float().t())
 
     def rotary_key(self):
         """Layers with equal keys share one cos/sin table per step."""
@@ -260,31 +295,39 @@ class MaskedAttention(torch.nn.Module):
         """conv_tail [slots, taps-1, q+k+v channels] fp32 (the cache
         manager's per-sequence state) is required when conv_taps > 0."""
         mc = self.mc
-        key = self.rotary_key()
-        cos_sin = tables.get(key) if tables is not None else None
-        if cos_sin is None:
-            cos_sin = ops.rotary_table(md.positions, self.rot_freqs,
-                                       self.rot_amp)
-            if tables is not None:
-                tables[key] = cos_sin
+        cos_sin = None
+        if not mc.plain_qk:
+            key = self.rotary_key()
+            cos_sin = tables.get(key) if tables is not None else None
+            if cos_sin is None:
+                cos_sin = ops.rotary_table(md.positions, self.rot_freqs,
+                                           self.rot_amp)
+                if tables is not None:
+                    tables[key] = cos_sin
         T, H, G = h.size(0), mc.heads, mc.kv_heads
+        own_kv = mc.kv_from is None
         proj = ops.linear(h, self.w_in, bias=self.b_in)
         k0, v0 = self.q_sz, self.q_sz + self.k_sz
-        g0 = v0 + self.v_sz
+        c_end = v0 + self.v_sz
+        g0 = self.gate_off
         qkv = proj
         if mc.conv_taps > 0:
-            qkv = torch.empty(T, g0, dtype=h.dtype, device=h.device)
+            qkv = torch.empty(T, c_end, dtype=h.dtype, device=h.device)
             ops.short_conv_state(
-                qkv, proj[:, :g0], self.w_conv, conv_tail, md.state_slots,
+                qkv, proj[:, :c_end], self.w_conv, conv_tail, md.state_slots,
                 md.seq_lens, md.query_starts if md.is_prefill else None,
                 md.query_lens if md.is_prefill else None)
         # strided views into the GEMM output: the kernels take row strides
         q = qkv[:, :k0].view(T, H, mc.dim)
-        k = qkv[:, k0:v0].view(T, G, mc.dim)
-        v = qkv[:, v0:g0].view(T, G, mc.vdim)
-        ops.rotary_norm_append(q, k, v, k_cache, v_cache, cos_sin,
-                               md.slot_mapping, self.eps, self.q_norm,
-                               self.k_norm, mc.norm_first)
+        if own_kv:
+            k = qkv[:, k0:v0].view(T, G, mc.dim)
+            v = qkv[:, v0:c_end].view(T, G, mc.vdim)
+            if mc.plain_qk:
+                ops.kv_append(k, v, k_cache, v_cache, md.slot_mapping)
+            else:
+                ops.rotary_norm_append(q, k, v, k_cache, v_cache, cos_sin,
+                                       md.slot_mapping, self.eps, self.q_norm,
+                                       self.k_norm, mc.norm_first)
         out = torch.empty(T, H, mc.vdim, dtype=h.dtype, device=h.device)
         ops.masked_attention(
             out, q, k_cache, v_cache, md.page_table, md.seq_lens,
@@ -293,8 +336,15 @@ class MaskedAttention(torch.nn.Module):
             mc.scale, mc.mask_kind, mc.mask_size, mc.keep_first,
             mc.sigmoid_weights, mc.softcap, self.key_bias,
             proj[:, g0:g0 + H] if mc.head_gate else None,
-            max_qlen=md.max_qlen if md.is_prefill else 1)
-        return ops.linear(out.view(T, H * mc.vdim), self.w_o)
+            max_qlen=md.max_qlen if md.is_prefill else 1,
+            dist_bias=self.dist_bias)
+        out = out.view(T, H * mc.vdim)
+        if mc.elem_gate:
+            ops.sigmoid_gate_rows(out, out, proj[:, g0:g0 + self.gate_sz])
+        y = ops.linear(out, self.w_o)
+        if self.extra_rows:
+            return y, proj[:, self.extra_off:self.extra_off + self.extra_rows]
+        return y
 
 
 class PolyNormFeedForward(torch.nn.Module):

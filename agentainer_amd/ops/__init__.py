@@ -639,7 +639,10 @@ def masked_attention(out, q, k_cache, v_cache, page_table, seq_lens,
                      query_starts, query_lens, scale: float, mask_kind: int,
                      mask_size: int, keep_first: int = 0,
                      sigmoid_weights: bool = False, softcap: float = 0.0,
-                     key_bias=None, head_gate=None, max_qlen: int = 1):
+                     key_bias=None, head_gate=None, max_qlen: int = 1,
+                     dist_bias=None):
+    """dist_bias: fp32 [H, 2] = (r1, r2) per head; r1 * ln(1 + r2 * distance)
+    is taken off every score (see reference.masked_attention)."""
     mod = _dispatch_masked("masked_attention", q)
     if mod:
         mod.masked_attention(out, q, k_cache, v_cache, page_table, seq_lens,
@@ -647,13 +650,13 @@ def masked_attention(out, q, k_cache, v_cache, page_table, seq_lens,
                              int(mask_kind), int(mask_size), int(keep_first),
                              bool(sigmoid_weights), float(softcap), key_bias,
                              head_gate, int(max_qlen), bool(MASKED_SIMPLE),
-                             int(MASKED_SPLITS))
+                             int(MASKED_SPLITS), dist_bias)
     else:
         reference.masked_attention(out, q, k_cache, v_cache, page_table,
                                    seq_lens, query_starts, query_lens, scale,
                                    mask_kind, mask_size, keep_first,
                                    sigmoid_weights, softcap, key_bias,
-                                   head_gate)
+                                   head_gate, dist_bias)
     return out
 
 
@@ -801,4 +804,161 @@ def routed_clamped_glu(out, gu, weight, n_experts: int, limit: float,
                                float(slope))
     else:
         reference.routed_clamped_glu(out, gu, weight, n_experts, limit, slope)
+    return out
+
+
+# ---------------------------------------------------------------------
+# Hashed bigram embedding, sigmoid-gated residual + layer norm, xIELU,
+# token-side gate, sigmoid group-limited routing, output-weighted gated
+# experts with a tail expert, latent rotary append, plain K/V append and
+# an elementwise output gate. Own extension (_hip_gated.so), same policy:
+# required on a GPU, fp32 torch references on CPU.
+# ---------------------------------------------------------------------
+
+_gated = None
+_gated_err: Optional[str] = None
+
+
+def _load_gated():
+    global _gated, _gated_err
+    if _gated is not None or _gated_err is not None:
+        return _gated
+    so = os.path.join(os.path.dirname(__file__), "_hip_gated.so")
+    if not os.path.exists(so):
+        _gated_err = (f"HIP extension not built ({so} missing); run "
+                      "python -m agentainer_amd.ops.build gated")
+        return None
+    try:
+        import importlib.util
+
+        spec = importlib.util.spec_from_file_location(
+            "agentainer_amd.ops._hip_gated", so)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _gated = mod
+    except Exception as exc:  # noqa: BLE001
+        _gated_err = f"HIP extension failed to load: {exc}"
+    return _gated
+
+
+def gated_available() -> bool:
+    return _load_gated() is not None
+
+
+def _dispatch_gated(name: str, t: torch.Tensor):
+    if t.is_cuda:
+        mod = _load_gated()
+        if mod is None:
+            raise RuntimeError(
+                f"op {name!r} on GPU requires the gfx950 HIP extension: "
+                f"{_gated_err}")
+        return mod
+    return None
+
+
+UPDATE_NONE = reference.UPDATE_NONE
+UPDATE_SIGMOID_GATE = reference.UPDATE_SIGMOID_GATE
+UPDATE_UNIT_RMS = reference.UPDATE_UNIT_RMS
+
+
+def bigram_embed(x_out, ids, embed, bigram, scale: float, mul_prev: int,
+                 mul_cur: int, buckets: int, prev_state, state_slots,
+                 seq_lens, query_starts, query_lens):
+    mod = _dispatch_gated("bigram_embed", x_out)
+    if mod:
+        mod.bigram_embed(x_out, ids, embed, bigram, float(scale),
+                         int(mul_prev), int(mul_cur), int(buckets),
+                         prev_state, state_slots, seq_lens, query_starts,
+                         query_lens)
+    else:
+        reference.bigram_embed(x_out, ids, embed, bigram, scale, mul_prev,
+                               mul_cur, buckets, prev_state, state_slots,
+                               seq_lens, query_starts, query_lens)
+    return x_out
+
+
+def residual_update_norm(x_res, y, update: int, gate, gate_bias, rms_w,
+                         eps: float, norm_w, norm_b, h_out):
+    mod = _dispatch_gated("residual_update_norm", x_res)
+    if mod:
+        mod.residual_update_norm(x_res, y, int(update), gate, gate_bias,
+                                 rms_w, float(eps), norm_w, norm_b, h_out)
+    else:
+        reference.residual_update_norm(x_res, y, update, gate, gate_bias,
+                                       rms_w, eps, norm_w, norm_b, h_out)
+    return h_out
+
+
+def xielu(out, z, coef):
+    mod = _dispatch_gated("xielu", z)
+    if mod:
+        mod.xielu(out, z, coef)
+    else:
+        reference.xielu(out, z, coef)
+    return out
+
+
+def gelu_gate_rows(out, t, table, ids, col0: int):
+    mod = _dispatch_gated("gelu_gate_rows", t)
+    if mod:
+        mod.gelu_gate_rows(out, t, table, ids, int(col0))
+    else:
+        reference.gelu_gate_rows(out, t, table, ids, col0)
+    return out
+
+
+def grouped_sigmoid_route(weight, logits, correction, n_experts: int,
+                          top: int, n_groups: int, keep_groups: int,
+                          group_top: int = 2):
+    mod = _dispatch_gated("grouped_sigmoid_route", logits)
+    if mod:
+        mod.grouped_sigmoid_route(weight, logits, correction, int(n_experts),
+                                  int(top), int(n_groups), int(keep_groups),
+                                  int(group_top))
+    else:
+        reference.grouped_sigmoid_route(weight, logits, correction, n_experts,
+                                        top, n_groups, keep_groups, group_top)
+    return weight
+
+
+def routed_silu_glu(out, gu, weight, n_experts: int, ff: int,
+                    tail_ff: int = 0):
+    mod = _dispatch_gated("routed_silu_glu", gu)
+    if mod:
+        mod.routed_silu_glu(out, gu, weight, int(n_experts), int(ff),
+                            int(tail_ff))
+    else:
+        reference.routed_silu_glu(out, gu, weight, n_experts, ff, tail_ff)
+    return out
+
+
+def latent_rotary_append(proj, heads: int, q_head: int, q_rot_off: int,
+                         kv_off: int, kv_rank: int, rot_dim: int, w_kv,
+                         eps: float, cos_sin, cache, slot_mapping):
+    mod = _dispatch_gated("latent_rotary_append", proj)
+    if mod:
+        mod.latent_rotary_append(proj, int(heads), int(q_head),
+                                 int(q_rot_off), int(kv_off), int(kv_rank),
+                                 int(rot_dim), w_kv, float(eps), cos_sin,
+                                 cache, slot_mapping)
+    else:
+        reference.latent_rotary_append(proj, heads, q_head, q_rot_off, kv_off,
+                                       kv_rank, rot_dim, w_kv, eps, cos_sin,
+                                       cache, slot_mapping)
+
+
+def kv_append(k, v, k_cache, v_cache, slot_mapping):
+    mod = _dispatch_gated("kv_append", k)
+    if mod:
+        mod.kv_append(k, v, k_cache, v_cache, slot_mapping)
+    else:
+        reference.kv_append(k, v, k_cache, v_cache, slot_mapping)
+
+
+def sigmoid_gate_rows(out, a, gate):
+    mod = _dispatch_gated("sigmoid_gate_rows", a)
+    if mod:
+        mod.sigmoid_gate_rows(out, a, gate)
+    else:
+        reference.sigmoid_gate_rows(out, a, gate)
     return out

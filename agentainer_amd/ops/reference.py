@@ -458,7 +458,8 @@ def masked_attention(out: torch.Tensor, q: torch.Tensor,
                      page_table: torch.Tensor, seq_lens: torch.Tensor,
                      query_starts, query_lens, scale: float, mask_kind: int,
                      mask_size: int, keep_first: int, sigmoid_weights: bool,
-                     softcap: float, key_bias, head_gate) -> None:
+                     softcap: float, key_bias, head_gate,
+                     dist_bias=None) -> None:
     """Grouped-query attention over paged per-head K/V pools.
 
     out [T, H, Dv], q [T, H, D]; query head h reads kv head h // (H/G).
@@ -467,7 +468,9 @@ def masked_attention(out: torch.Tensor, q: torch.Tensor,
     sigmoid_weights) sigmoid(score + key_bias[h]) per visible key without
     normalization. head_gate [T, H], when given, multiplies head h's
     output by sigmoid(head_gate[t, h]). query_starts/query_lens None means
-    one new token per sequence; rows with seq_len <= 0 come back zero."""
+    one new token per sequence; rows with seq_len <= 0 come back zero.
+    dist_bias fp32 [H, 2] = (r1, r2) per head takes r1 * ln(1 + r2 * (p - j))
+    off the (capped) score of key j for the query at position p."""
     H = q.size(1)
     G, PS = k_cache.size(1), k_cache.size(2)
     rep = H // G
@@ -491,6 +494,11 @@ def masked_attention(out: torch.Tensor, q: torch.Tensor,
         qpos = (total - qlen + torch.arange(qlen)).view(1, qlen, 1)
         seen = mask_visible(qpos, pos.view(1, 1, -1), mask_kind, mask_size,
                             keep_first)
+        if dist_bias is not None:
+            db = dist_bias.float()
+            dist = (qpos - pos.view(1, 1, -1)).clamp(min=0).float()
+            s = s - db[:, 0].view(H, 1, 1) * torch.log1p(
+                db[:, 1].view(H, 1, 1) * dist)
         if sigmoid_weights:
             if key_bias is not None:
                 s = s + key_bias.float().view(H, 1, 1)
@@ -721,3 +729,189 @@ def routed_clamped_glu(out: torch.Tensor, gu: torch.Tensor,
     y = g * torch.sigmoid(slope * g) * (u + 1.0) * w
     y = torch.where(w == 0, torch.zeros_like(y), y)
     out.copy_(y.view(T, E * F_).to(out.dtype))
+
+
+# ---------------------------------------------------------------------
+# Hashed bigram embedding, sigmoid-gated residual with layer norm, xIELU,
+# token-side gate, sigmoid group-limited routing with always-on experts,
+# output-weighted gated experts with an odd-sized tail expert, latent
+# rotary append, plain K/V append, elementwise output gate.
+# ---------------------------------------------------------------------
+
+UPDATE_NONE, UPDATE_SIGMOID_GATE, UPDATE_UNIT_RMS = 0, 1, 2
+
+
+def bigram_embed(x_out: torch.Tensor, ids: torch.Tensor, embed: torch.Tensor,
+                 bigram, scale: float, mul_prev: int, mul_cur: int,
+                 buckets: int, prev_state, state_slots, seq_lens,
+                 query_starts, query_lens) -> None:
+    """x_out (fp32 [T, W]) = scale * embed[id] + bigram[row], row =
+    (mul_prev * previous id + mul_cur * id) mod buckets; a sequence's first
+    token (position 0) takes row `buckets`. The previous id of a portion's
+    first row comes from prev_state [slots] (int32), which is rewritten
+    with the portion's last id. bigram None: plain scaled embedding."""
+    x_out.copy_(embed[ids].float() * scale)
+    if bigram is None:
+        return
+    for b in range(seq_lens.numel()):
+        s0, n, pos0 = _step_rows(b, seq_lens, query_starts, query_lens)
+        if n <= 0:
+            continue
+        slot = int(state_slots[b])
+        prev = int(prev_state[slot])
+        for r in range(s0, s0 + n):
+            tok = int(ids[r])
+            if r == s0 and pos0 <= 0:
+                row = buckets
+            else:
+                row = (prev * mul_prev + tok * mul_cur) % buckets
+            x_out[r] += bigram[row].float()
+            prev = tok
+        prev_state[slot] = prev
+
+
+def residual_update_norm(x_res: torch.Tensor, y, update: int, gate, gate_bias,
+                         rms_w, eps: float, norm_w, norm_b,
+                         h_out) -> None:
+    """fp32 residual update fused with the norm that feeds the next GEMM.
+    update: NONE; SIGMOID_GATE x += sigmoid(gate + gate_bias) * y;
+    UNIT_RMS x += y / sqrt(mean(y^2) + eps) * rms_w. Then h_out = layer
+    norm of x ((x - mean) / sqrt(var + eps) * norm_w + norm_b), or just x
+    in h_out's dtype when norm_w is None; h_out None skips it."""
+    if update == UPDATE_SIGMOID_GATE:
+        g = gate.float()
+        if gate_bias is not None:
+            g = g + gate_bias.float()
+        x_res.add_(torch.sigmoid(g) * y.float())
+    elif update == UPDATE_UNIT_RMS:
+        x_res.add_(_unit(y.float(), eps) * rms_w.float())
+    if h_out is None:
+        return
+    if norm_w is None:
+        h_out.copy_(x_res.to(h_out.dtype))
+        return
+    d = x_res - x_res.mean(-1, keepdim=True)
+    r = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps)
+    r = r * norm_w.float()
+    if norm_b is not None:
+        r = r + norm_b.float()
+    h_out.copy_(r.to(h_out.dtype))
+
+
+def xielu(out: torch.Tensor, z: torch.Tensor, coef: torch.Tensor) -> None:
+    """coef = (a_pos, a_neg) fp32: z > 0 -> a_pos z^2 + z/2; z <= 0 ->
+    a_neg (e^z - 1 - z) + z/2."""
+    zf = z.float()
+    zn = zf.clamp(max=0.0)
+    out.copy_(torch.where(zf > 0, coef[0] * zf * zf + 0.5 * zf,
+                          coef[1] * (torch.expm1(zn) - zn) + 0.5 * zn
+                          ).to(out.dtype))
+
+
+def gelu_gate_rows(out: torch.Tensor, t: torch.Tensor, table: torch.Tensor,
+                   ids: torch.Tensor, col0: int) -> None:
+    """out[r, d] = gelu_tanh(t[r, d]) * table[ids[r], col0 + d]."""
+    z = t.float()
+    g = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654
+                                    * (z + 0.044715 * z * z * z)))
+    e = table[ids, col0:col0 + t.size(1)].float()
+    out.copy_((g * e).to(out.dtype))
+
+
+def grouped_sigmoid_route(weight: torch.Tensor, logits: torch.Tensor,
+                          correction, n_experts: int, top: int, n_groups: int,
+                          keep_groups: int, group_top: int) -> None:
+    """Dense routing weights [T, E + A] (0 = not chosen), fp32 throughout.
+    s = sigmoid(logits); choice score c = s + correction (columns < E);
+    experts form n_groups equal consecutive groups, a group scores the sum
+    of its group_top largest c and only the keep_groups best groups stay
+    eligible (the others count as -inf); the `top` eligible experts with
+    the largest c weigh s, not renormalized. Columns >= E are always-on
+    gates: weight = sigmoid(logit)."""
+    T, E = logits.size(0), n_experts
+    s_all = torch.sigmoid(logits.float())
+    s = s_all[:, :E]
+    c = s if correction is None else s + correction.float()
+    if n_groups > 1 and keep_groups < n_groups:
+        per = E // n_groups
+        gs = c.view(T, n_groups, per).topk(min(group_top, per), dim=-1
+                                           ).values.sum(-1)
+        keep = torch.zeros(T, n_groups, dtype=torch.bool)
+        keep.scatter_(1, gs.topk(keep_groups, dim=-1).indices, True)
+        ok = keep.unsqueeze(-1).expand(T, n_groups, per)
+        c = c.masked_fill(~ok.reshape(T, E), float("-inf"))
+    idx = c.topk(top, dim=-1).indices
+    weight.zero_()
+    weight[:, :E].scatter_(1, idx, s.gather(1, idx))
+    weight[:, E:] = s_all[:, E:]
+
+
+def routed_silu_glu(out: torch.Tensor, gu: torch.Tensor, weight: torch.Tensor,
+                    n_experts: int, ff: int, tail_ff: int) -> None:
+    """Stacked gated experts with the routing weight on the OUTPUT side.
+    gu [T, E*2F + 2Ft]: expert e owns gate | up at e*2F; a tail expert of
+    inner size Ft (0 = none) follows at E*2F and is weighed by weight[:, E].
+    out[t, e*F + f] = weight[t, e] * silu(gate) * up, 0 where the weight is
+    0; out [T, E*F + Ft]."""
+    T, E, F_ = gu.size(0), n_experts, ff
+    g3 = gu[:, :E * 2 * F_].reshape(T, E, 2 * F_).float()
+    g, u = g3[..., :F_], g3[..., F_:]
+    w = weight[:, :E].float().unsqueeze(-1)
+    y = g * torch.sigmoid(g) * u * w
+    y = torch.where(w == 0, torch.zeros_like(y), y)
+    out[:, :E * F_] = y.view(T, E * F_).to(out.dtype)
+    if tail_ff > 0:
+        tg = gu[:, E * 2 * F_:E * 2 * F_ + tail_ff].float()
+        tu = gu[:, E * 2 * F_ + tail_ff:E * 2 * F_ + 2 * tail_ff].float()
+        out[:, E * F_:] = (tg * torch.sigmoid(tg) * tu
+                           * weight[:, E:E + 1].float()).to(out.dtype)
+
+
+def latent_rotary_append(proj: torch.Tensor, heads: int, q_head: int,
+                         q_rot_off: int, kv_off: int, kv_rank: int,
+                         rot_dim: int, w_kv: torch.Tensor, eps: float,
+                         cos_sin: torch.Tensor, cache: torch.Tensor,
+                         slot_mapping: torch.Tensor) -> None:
+    """One step's rows of a latent-attention input projection:
+    proj[:, h*q_head + q_rot_off : +rot_dim] (every query head's rotated
+    part) is rotated IN PLACE; proj[:, kv_off : kv_off+kv_rank] is
+    RMS-normed with w_kv into cache[slot, :kv_rank]; the shared key part
+    proj[:, kv_off+kv_rank : +rot_dim] is rotated into cache[slot,
+    kv_rank : kv_rank+rot_dim]; the pool's remaining columns are zeroed.
+    Rotation pairs coordinate i with i + half (cos_sin [T, 2*half] from
+    rotary_table, 2*half <= rot_dim; the rest passes). slot < 0 skips the
+    append."""
+    T = proj.size(0)
+    q = proj[:, :heads * q_head].view(T, heads, q_head)
+    qr = q[:, :, q_rot_off:q_rot_off + rot_dim]
+    qr.copy_(_rotate_half(qr.float(), cos_sin).to(proj.dtype))
+    c = proj[:, kv_off:kv_off + kv_rank].float()
+    c = (_unit(c, eps) * w_kv.float()).to(cache.dtype)
+    kr = proj[:, kv_off + kv_rank:kv_off + kv_rank + rot_dim].float()
+    kr = _rotate_half(kr.unsqueeze(1), cos_sin).squeeze(1).to(cache.dtype)
+    Rp = cache.size(2)
+    flat = cache.view(-1, Rp)
+    ok = slot_mapping >= 0
+    rows = slot_mapping[ok].long()
+    flat[rows, :kv_rank] = c[ok]
+    flat[rows, kv_rank:kv_rank + rot_dim] = kr[ok]
+    if Rp > kv_rank + rot_dim:
+        flat[rows, kv_rank + rot_dim:] = 0
+
+
+def kv_append(k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
+              v_cache: torch.Tensor, slot_mapping: torch.Tensor) -> None:
+    """k [T, G, D], v [T, G, Dv] -> pools [P, G, PS, D] / [P, G, PS, Dv] at
+    slot = page*PS + offset (slot < 0 skips)."""
+    PS = k_cache.size(2)
+    ok = slot_mapping >= 0
+    rows = slot_mapping[ok].long()
+    page, off = rows // PS, rows % PS
+    k_cache[page, :, off] = k[ok].to(k_cache.dtype)
+    v_cache[page, :, off] = v[ok].to(v_cache.dtype)
+
+
+def sigmoid_gate_rows(out: torch.Tensor, a: torch.Tensor,
+                      gate: torch.Tensor) -> None:
+    """out[t, c] = a[t, c] * sigmoid(gate[t, c])."""
+    out.copy_((a.float() * torch.sigmoid(gate.float())).to(out.dtype))
