@@ -494,7 +494,7 @@ class GroupedSigmoidExperts(torch.nn.Module):
             ops.routed_silu_glu(act, gu, w, 1, Fh, 0)
             out.index_add_(0, rows, ops.linear(
                 act, self.down[:, e * Fh:(e + 1) * Fh]).float())
-        return out, dense[:, extra0:extra0 + self.extra_rows]
+        return out.to(h.dtype), dense[:, extra0:extra0 + self.extra_rows]
 
 
 class SipelornLayer(torch.nn.Module):

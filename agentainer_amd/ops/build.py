@@ -61,6 +61,16 @@ RECURRENT_SOURCES = [
     "grouped_route.hip",
 ]
 
+# hashed bigram embedding, gated residual + layer norm, xIELU, sigmoid
+# group routing, output-weighted gated experts, latent rotary append
+GATED_SOURCES = [
+    "gated_bindings.cpp",
+    "gated_norm.hip",
+    "bigram_embed.hip",
+    "sigmoid_route.hip",
+    "latent_rotary.hip",
+]
+
 SOURCES = [
     "bindings.cpp",
     "rmsnorm.hip",
@@ -95,6 +105,11 @@ def _target(target: str):
         return (os.path.join(HERE, f"_hip_recurrent{sfx}.so"),
                 os.path.join(HERE, "_build_recurrent" + sfx),
                 RECURRENT_SOURCES, "_hip_recurrent")
+    if target == "gated":
+        sfx = "_asan" if ASAN else ""
+        return (os.path.join(HERE, f"_hip_gated{sfx}.so"),
+                os.path.join(HERE, "_build_gated" + sfx), GATED_SOURCES,
+                "_hip_gated")
     if target != "core":
         raise ValueError(f"unknown build target {target!r}")
     return OUT, OBJ_DIR, SOURCES, "_hip_ops"
@@ -115,7 +130,7 @@ def needs_build(target: str = "core") -> bool:
 def build(verbose: bool = True, force: bool = False,
           target: str = "core") -> str:
     if target == "all":
-        target = "core+latent+masked+recurrent"
+        target = "core+latent+masked+recurrent+gated"
     if "+" in target:
         out = ""
         for t in target.split("+"):

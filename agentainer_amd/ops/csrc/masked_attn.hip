@@ -5,6 +5,7 @@
 //   q [T, H, D], out [T, H, Dv]; query head h reads kv head h / (H/G).
 //
 //   score  = <q, k> * scale;  score <- cap * tanh(score / cap)   (cap > 0)
+//            score <- score - r1[h] * ln(1 + r2[h] * (p - j))    (dist given)
 //   mask   : causal   j <= p
 //            window   j <= p and (p - j < size  or  j < keep)
 //            chunk    j <= p and floor(p/size) == floor(j/size)
@@ -70,6 +71,15 @@ __device__ __forceinline__ float fast_tanh(float x) {
   return 2.0f * fast_sigmoid(2.0f * x) - 1.0f;
 }
 
+// distance bias: r1 * ln(1 + r2 * d), d >= 0
+__device__ __forceinline__ float dist_penalty(float r1, float r2, int d) {
+  return r1 * log1pf(r2 * (float)max(d, 0));
+}
+// tile kernels: hardware log2 (the argument is >= 1)
+__device__ __forceinline__ float fast_dist_penalty(float r1, float r2, int d) {
+  return r1 * 0.6931471805599453f * __log2f(fmaf(r2, (float)max(d, 0), 1.0f));
+}
+
 // token position -> (page index in the sequence's table, row in the page);
 // page sizes that are powers of two (ps_shift >= 0) avoid the division
 __device__ __forceinline__ void page_of(int j, int PS, int ps_shift, int& pg,
@@ -103,7 +113,8 @@ __global__ __launch_bounds__(64) void masked_attn_rowwave_kernel(
     const int* __restrict__ q_starts, const int* __restrict__ q_lens,
     float scale, int kind, int size, int keep, int sigmoid_w, float softcap,
     const float* __restrict__ key_bias, const T* __restrict__ gate, long g_ts,
-    int H, int G, int D, int Dv, int PS, int max_pages, int vec) {
+    const float* __restrict__ dist, int H, int G, int D, int Dv, int PS,
+    int max_pages, int vec) {
   extern __shared__ float smem[];
   float* q_s = smem;       // [D]
   float* p_s = smem + D;   // [64]
@@ -128,6 +139,7 @@ __global__ __launch_bounds__(64) void masked_attn_rowwave_kernel(
   __syncthreads();
   const int* pt = page_table + (long)b * max_pages;
   const float bias = (sigmoid_w && key_bias != nullptr) ? key_bias[h] : 0.f;
+  const float r1 = dist ? dist[2 * h] : 0.f, r2 = dist ? dist[2 * h + 1] : 0.f;
 
   float m = -FLT_MAX, l = 0.f;
   float acc[RW_MAX_ACC];
@@ -156,6 +168,7 @@ __global__ __launch_bounds__(64) void masked_attn_rowwave_kernel(
       }
       s = d * scale;
       if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      if (dist) s -= dist_penalty(r1, r2, qpos - j);
     }
     float p, alpha = 1.0f;
     if (sigmoid_w) {
@@ -219,8 +232,8 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
     const int* __restrict__ seq_lens, const int* __restrict__ q_starts,
     const int* __restrict__ q_lens, float scale, int kind, int size, int keep,
     int sigmoid_w, float softcap, const float* __restrict__ key_bias,
-    const short* __restrict__ gate, long g_ts, int H, int G, int nd, int nv,
-    int PS, int max_pages, int ps_shift) {
+    const short* __restrict__ gate, long g_ts, const float* __restrict__ dist,
+    int H, int G, int nd, int nv, int PS, int max_pages, int ps_shift) {
   extern __shared__ __attribute__((aligned(16))) short lds[];
   constexpr int KL = NDB / 2;              // 16-byte K loads per thread
   const int D = nd * 32, Dv = nv * 16;
@@ -276,6 +289,7 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
   const int wq_last = ctx + min(cw0 + COLS_PER_WAVE - 1, ncols - 1) / R;
   const int w_lo = mask_lo(wq_first, kind, size);
   const float bias = (sigmoid_w && key_bias != nullptr) ? key_bias[h] : 0.f;
+  const float r1 = dist ? dist[2 * h] : 0.f, r2 = dist ? dist[2 * h + 1] : 0.f;
 
   // Q^T as the first MFMA's B operand: lane -> column l16, dims c*32+lg*8..
   bf16v8 qf[NDB];
@@ -389,6 +403,7 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
         vis[e] = j <= qpos && (j >= lo || j < keep);
         float s = sv[e] * scale;
         if (softcap > 0.f) s = softcap * fast_tanh(s * inv_cap);
+        if (dist) s -= fast_dist_penalty(r1, r2, qpos - j);
         sv[e] = s;
       }
       float pv[8];
@@ -480,9 +495,9 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
     const short* __restrict__ vc, const int* __restrict__ page_table,
     const int* __restrict__ seq_lens, float scale, int kind, int size, int keep,
     int sigmoid_w, float softcap, const float* __restrict__ key_bias,
-    const short* __restrict__ gate, long g_ts, int H, int G, int nd, int nv,
-    int PS, int max_pages, int ps_shift, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int n_splits) {
+    const short* __restrict__ gate, long g_ts, const float* __restrict__ dist,
+    int H, int G, int nd, int nv, int PS, int max_pages, int ps_shift,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits) {
   extern __shared__ __attribute__((aligned(16))) short lds[];
   const int D = nd * 32, Dv = nv * 16;
   const int split = blockIdx.x, b = blockIdx.y, g = blockIdx.z;
@@ -520,6 +535,7 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
   const bool col_ok = l16 < R;
   const int h = g * R + (col_ok ? l16 : 0);
   const float bias = (sigmoid_w && key_bias != nullptr) ? key_bias[h] : 0.f;
+  const float r1 = dist ? dist[2 * h] : 0.f, r2 = dist ? dist[2 * h + 1] : 0.f;
   const int cq = col_ok ? qpos : -1;
 
   bf16v8 qf[NDB];
@@ -645,6 +661,7 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
       vis[e] = j <= cq && (j >= lo || j < keep);
       float s = sv[e] * scale;
       if (softcap > 0.f) s = softcap * fast_tanh(s * inv_cap);
+      if (dist) s -= fast_dist_penalty(r1, r2, qpos - j);
       sv[e] = s;
     }
     if (sigmoid_w) {
@@ -776,7 +793,8 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                       bool sigmoid_weights, double softcap,
                       c10::optional<torch::Tensor> key_bias,
                       c10::optional<torch::Tensor> head_gate, long max_qlen,
-                      bool force_simple, long splits) {
+                      bool force_simple, long splits,
+                      c10::optional<torch::Tensor> dist_bias) {
   TORCH_CHECK(q.dim() == 3 && out.dim() == 3 && q.stride(2) == 1 &&
               out.stride(2) == 1);
   const int T_ = q.size(0), H = q.size(1), D = q.size(2), Dv = out.size(2);
@@ -827,6 +845,13 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                 head_gate->scalar_type() == q.scalar_type());
     g_ts = head_gate->stride(0);
   }
+  const float* db = nullptr;
+  if (dist_bias.has_value()) {
+    TORCH_CHECK(dist_bias->scalar_type() == at::kFloat &&
+                dist_bias->numel() == 2 * H && dist_bias->is_contiguous(),
+                "dist_bias is fp32 [heads, 2]");
+    db = dist_bias->data_ptr<float>();
+  }
   if (T_ == 0 || B == 0) return;
   const int keep = mask_kind == MK_WINDOW ? (int)keep_first : 0;
   auto stream = at::hip::getCurrentHIPStream();
@@ -874,8 +899,8 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                      (const short*)v_cache.data_ptr(),                        \
                      page_table.data_ptr<int>(), seq_lens.data_ptr<int>(),    \
                      (float)scale, (int)mask_kind, (int)mask_size, keep,      \
-                     sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts, H, \
-                     G, nd, nv, PS, max_pages, ps_shift, pop, pmlp,     \
+                     sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts,   \
+                     db, H, G, nd, nv, PS, max_pages, ps_shift, pop, pmlp,    \
                      (int)n_splits)
       if (nd <= 4 && nv <= 4) {
         LAUNCH_DECODE(4, 4);
@@ -905,8 +930,8 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                      (const short*)v_cache.data_ptr(),                        \
                      page_table.data_ptr<int>(), seq_lens.data_ptr<int>(), qs, \
                      ql, (float)scale, (int)mask_kind, (int)mask_size, keep,  \
-                     sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts, H, \
-                     G, nd, nv, PS, max_pages, ps_shift)
+                     sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts,   \
+                     db, H, G, nd, nv, PS, max_pages, ps_shift)
     if (nd <= 4 && nv <= 4) {
       LAUNCH_MFMA(4, 4);
     } else if (nd <= 4 && nv <= 8) {
@@ -933,7 +958,7 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
         (const T*)k_cache.data_ptr(), (const T*)v_cache.data_ptr(),
         page_table.data_ptr<int>(), seq_lens.data_ptr<int>(), qs, ql,
         (float)scale, (int)mask_kind, (int)mask_size, keep,
-        sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts, H, G, D, Dv, PS,
-        max_pages, vec);
+        sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts, db, H, G, D, Dv,
+        PS, max_pages, vec);
   });
 }

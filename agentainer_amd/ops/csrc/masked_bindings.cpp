@@ -24,7 +24,8 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                       bool sigmoid_weights, double softcap,
                       c10::optional<torch::Tensor> key_bias,
                       c10::optional<torch::Tensor> head_gate, long max_qlen,
-                      bool force_simple, long splits);
+                      bool force_simple, long splits,
+                      c10::optional<torch::Tensor> dist_bias);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "agentainer_amd CDNA4 (gfx950) masked-attention family kernels";
@@ -37,5 +38,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("rotary_norm_append", &rotary_norm_append,
         "rotary + q/k rms norm; append K/V to the paged pools");
   m.def("masked_attention", &masked_attention,
-        "chunk / window masked GQA with softmax or sigmoid weights");
+        "chunk / window masked GQA with softmax or sigmoid weights and an "
+        "optional logarithmic distance bias");
 }
