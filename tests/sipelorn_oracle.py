@@ -149,25 +149,34 @@ def conv_keys_values(h, w, p, mx):
     return k.view(T, G, D), v.view(T, G, Dv)
 
 
+def biased_window_softmax(q, k, v, scale, size, r1, r2):
+    """q [T, H, D], k [T, G, D], v [T, G, Dv]; query i of head hd sees keys
+    j with 0 <= i - j < size and scores q.k * scale - r1[hd] ln(1 + r2[hd]
+    (i - j)); softmax over the seen keys. Returns [T, H, Dv]."""
+    T, H = q.shape[0], q.shape[1]
+    G = k.shape[1]
+    out = torch.zeros(T, H, v.shape[2], dtype=F64)
+    for hd in range(H):
+        g = hd // (H // G)
+        for i in range(T):
+            j0 = max(0, i - size + 1)
+            dist = torch.arange(i - j0, -1, -1, dtype=F64)      # i - j
+            sc = (k[j0:i + 1, g] @ q[i, hd]) * scale \
+                - float(r1[hd]) * torch.log1p(float(r2[hd]) * dist)
+            out[i, hd] = torch.softmax(sc, dim=0) @ v[j0:i + 1, g]
+    return out
+
+
 def window_attention(h, w, p, mx, kv=None):
     """kv: (k, v) borrowed from another layer, or None to make its own.
     Returns (mixer output, (k, v))."""
     T = h.shape[0]
-    H, G, D, Dv = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
-    size = int(mx["mask"]["size"])
+    H, D, Dv = mx["heads"], mx["dim"], mx["vdim"]
     q = causal_conv(h @ w[p + "q"].T + w[p + "q.b"],
                     w[p + "q.conv"]).view(T, H, D)
     k, v = kv if kv is not None else conv_keys_values(h, w, p, mx)
-    out = torch.zeros(T, H, Dv, dtype=F64)
-    for hd in range(H):
-        g = hd // (H // G)
-        r1, r2 = float(w[p + "r1"][hd]), float(w[p + "r2"][hd])
-        for i in range(T):
-            j0 = max(0, i - size + 1)
-            dist = torch.arange(i - j0, -1, -1, dtype=F64)      # i - j
-            sc = (k[j0:i + 1, g] @ q[i, hd]) * mx["scale"] \
-                - r1 * torch.log1p(r2 * dist)
-            out[i, hd] = torch.softmax(sc, dim=0) @ v[j0:i + 1, g]
+    out = biased_window_softmax(q, k, v, mx["scale"], int(mx["mask"]["size"]),
+                                w[p + "r1"], w[p + "r2"])
     gate = torch.sigmoid(h @ w[p + "g"].T)
     return (out.reshape(T, H * Dv) * gate) @ w[p + "o"].T, (k, v)
 
@@ -372,7 +381,7 @@ def random_weights(cfg: dict, seed: int = 0) -> Dict[str, torch.Tensor]:
                                                    generator=g) * 0.6
                                        ).bfloat16().float()
             w[p + "r1"] = vec(H, 0.6, 0.3).abs()
-            w[p + "r2"] = vec(H, 0.5, 0.2).abs() + 0.05
+            w[p + "r2"] = (vec(H, 0.5, 0.2).abs() + 0.05).bfloat16().float()
             w[p + "g"] = mat(H * Dv, W)
             w[p + "o"] = mat(W, H * Dv)
         else:
