@@ -58,6 +58,17 @@ __global__ __launch_bounds__(256) void bigram_embed_kernel(
     br = bigram + row * W;
   }
   float* xr = x + (long)r * W;
+  if (W % 4 == 0) {   // table rows then start 4-element aligned
+    for (int i = threadIdx.x * 4; i < W; i += 256 * 4) {
+      float v[4], b[4] = {0.f, 0.f, 0.f, 0.f};
+      ld4(er, i, v);
+      if (br) ld4(br, i, b);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = fmaf(v[j], scale, b[j]);
+      st4(xr, i, v);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < W; i += 256) {
     float v = ldf(er, i) * scale;
     if (br) v += ldf(br, i);

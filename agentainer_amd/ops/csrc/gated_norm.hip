@@ -152,6 +152,27 @@ __global__ __launch_bounds__(256) void residual_update_norm_kernel(
   }
 }
 
+// bf16, 8 values (16 bytes) per thread
+__global__ void xielu_bf16x8_kernel(short* __restrict__ out,
+                                    const short* __restrict__ z, long z_rs,
+                                    const float* __restrict__ coef, long n,
+                                    int C) {
+  const long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (i >= n) return;
+  const long r = i / C;
+  const int c = (int)(i % C);
+  const float ap = coef[0], an = coef[1];
+  const bf16x8 v = *reinterpret_cast<const bf16x8*>(z + r * z_rs + c);
+  bf16x8 o;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float a = bits2f(v[j]);
+    o[j] = f2bits(a > 0.f ? fmaf(ap * a, a, 0.5f * a)
+                          : fmaf(an, expm1f(a) - a, 0.5f * a));
+  }
+  *reinterpret_cast<bf16x8*>(out + i) = o;
+}
+
 template <typename T, int VEC>
 __global__ void xielu_kernel(T* __restrict__ out, const T* __restrict__ z,
                              long z_rs, const float* __restrict__ coef, long n,
@@ -305,6 +326,15 @@ void xielu(torch::Tensor out, torch::Tensor z, torch::Tensor coef) {
   if (n == 0) return;
   const bool vec = C % 4 == 0 && aligned_rows(z, 4);
   auto stream = at::hip::getCurrentHIPStream();
+  if (out.scalar_type() == at::kBFloat16 && C % 8 == 0 && aligned_rows(z, 8) &&
+      reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(z.data_ptr()) % 16 == 0) {
+    hipLaunchKernelGGL(xielu_bf16x8_kernel, dim3((n / 8 + 255) / 256),
+                       dim3(256), 0, stream, (short*)out.data_ptr(),
+                       (const short*)z.data_ptr(), (long)z.stride(0),
+                       coef.data_ptr<float>(), n, C);
+    return;
+  }
   LATENT_DISPATCH_T(out, {
     if (vec) {
       hipLaunchKernelGGL((xielu_kernel<T, 4>), dim3((n / 4 + 255) / 256),

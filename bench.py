@@ -86,7 +86,7 @@ def _parser():
                    help="--arch-compare: which size points to run "
                         "(default: all points of the design)")
     p.add_argument("--arch-design", default="lelitar",
-                   choices=["lelitar", "volalorn", "pekarax"],
+                   choices=["lelitar", "volalorn", "pekarax", "sipelorn"],
                    help="--arch-compare: which design to measure")
     return p
 
@@ -235,6 +235,71 @@ def _pekarax_points():
     }
 
 
+def _sipelorn_points():
+    """Sipelorn size points beside Mixtral stacks of equal width, attention
+    head counts, expert count, expert size and top-k: four layers (latent
+    attention, window attention, window attention on the previous layer's
+    keys and values, latent attention); three are followed by the routed
+    experts (two groups of which one is kept, plus a shared expert of a
+    quarter of an expert's size), the last by a dense xIELU feed-forward of
+    twice an expert's size. Bigram table, per-layer token inputs of 256
+    values and gated residuals as the design has them. The latent pool row
+    (latent + rotated key part) is 256 wide at width 2048 and 512 at 4096."""
+    from agentainer_amd import ops
+    from agentainer_amd.models.mixtral import MixtralConfig
+    from agentainer_amd.models.sipelorn import (RotaryLatentConfig,
+                                                SipelornConfig,
+                                                SipelornFeedForwardConfig,
+                                                SipelornLayerConfig)
+    from agentainer_amd.models.volalorn import MaskedAttentionConfig
+
+    def sip(name, width, heads, kv, ff, experts, top, rank, window):
+        moe = SipelornFeedForwardConfig("moe", ff, experts=experts, top=top,
+                                        groups=2, keep_groups=1,
+                                        shared_ff=ff // 4)
+        latent = RotaryLatentConfig(
+            heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=rank,
+            scale=192 ** -0.5, rot_dims=64, rot_base=1e6,
+            rot_scaling={"factor": 4.0, "original": 4096, "fast": 32.0,
+                         "slow": 1.0})
+
+        def attn(src=None):
+            return MaskedAttentionConfig(
+                heads=heads, kv_heads=kv, dim=128, vdim=128, scale=0.09,
+                mask_kind=ops.MASK_WINDOW, mask_size=window, qkv_bias=True,
+                conv_taps=4, plain_qk=True, dist_bias=True, elem_gate=True,
+                kv_from=src)
+
+        layers = [
+            SipelornLayerConfig("latent_attention", latent=latent, mlp=moe),
+            SipelornLayerConfig("attention", attn=attn(), mlp=moe),
+            SipelornLayerConfig("attention", attn=attn(1), mlp=moe),
+            SipelornLayerConfig("latent_attention", latent=latent,
+                                mlp=SipelornFeedForwardConfig("dense",
+                                                              2 * ff))]
+        return SipelornConfig(name=name, vocab_size=32000, hidden_size=width,
+                              layers=layers, norm_eps=1e-5, embed_scale=8.0,
+                              bigram_buckets=65521, bigram_mul_prev=36313,
+                              bigram_mul_cur=27191, side_dim=256)
+
+    return {
+        "s": ("w2048-8x4096-top2",
+              sip("sipelorn-s", 2048, 16, 4, 4096, 8, 2, 192, 1024),
+              MixtralConfig(name="mixtral-s", vocab_size=32000,
+                            hidden_size=2048, n_layers=4, n_heads=16,
+                            n_kv_heads=4, intermediate_size=4096,
+                            n_experts=8, top_k=2, tie_embeddings=False),
+              "mixtral"),
+        "l": ("w4096-8x7168-top2",
+              sip("sipelorn-l", 4096, 32, 8, 7168, 8, 2, 448, 4096),
+              MixtralConfig(name="mixtral-l", vocab_size=32000,
+                            hidden_size=4096, n_layers=4, n_heads=32,
+                            n_kv_heads=8, intermediate_size=7168,
+                            n_experts=8, top_k=2, tie_embeddings=False),
+              "mixtral"),
+    }
+
+
 def run_arch_compare(args):
     """Prefill (8 x 1024-token prompts per step) and decode (64 sequences at
     1024 tokens of context, captured graph) throughput, through the
@@ -243,6 +308,7 @@ def run_arch_compare(args):
     from agentainer_amd.models.lelitar import LelitarForCausalLM
     from agentainer_amd.models.mixtral import MixtralForCausalLM
     from agentainer_amd.models.pekarax import PekaraxForCausalLM
+    from agentainer_amd.models.sipelorn import SipelornForCausalLM
     from agentainer_amd.models.volalorn import VolalornForCausalLM
 
     dev = "cuda" if torch.cuda.is_available() else "cpu"
@@ -303,9 +369,10 @@ def run_arch_compare(args):
 
     design = args.arch_design
     pts = {"volalorn": _volalorn_points, "pekarax": _pekarax_points,
-           "lelitar": _arch_points}[design]()
+           "sipelorn": _sipelorn_points, "lelitar": _arch_points}[design]()
     ours_cls = {"volalorn": VolalornForCausalLM,
                 "pekarax": PekaraxForCausalLM,
+                "sipelorn": SipelornForCausalLM,
                 "lelitar": LelitarForCausalLM}[design]
     for key in (args.arch_sizes or ",".join(pts)).split(","):
         label, lcfg, rcfg, kind = pts[key.strip()]
