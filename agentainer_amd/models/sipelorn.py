@@ -152,7 +152,7 @@ class SipelornConfig:
         for i, l in enumerate(self.layers):
             d: Dict[str, tuple] = {}
             a = l.attn
-            if a is not None and a.conv_taps > 1:
+            if a is not None and a.conv_taps > 0:
                 ch = a.heads * a.dim
                 if a.kv_from is None:
                     ch += a.kv_heads * (a.dim + a.vdim)
@@ -187,7 +187,7 @@ def config_from_dict(d: dict, name: str = "sipelorn") -> SipelornConfig:
                 dim=int(mx["dim"]), vdim=int(mx["vdim"]),
                 scale=float(mx["scale"]), mask_kind=ops.MASK_WINDOW,
                 mask_size=int(mx["mask"]["size"]), qkv_bias=True,
-                conv_taps=int(mx.get("conv", 0)), plain_qk=True,
+                conv_taps=int(mx.get("conv") or 0), plain_qk=True,
                 dist_bias=True, elem_gate=True,
                 kv_from=None if src is None else int(src))
             a = lc.attn

@@ -260,8 +260,8 @@ def _sipelorn_points():
         latent = RotaryLatentConfig(
             heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=rank,
             scale=192 ** -0.5, rot_dims=64, rot_base=1e6,
-            rot_scaling={"factor": 4.0, "original": 4096, "fast": 32.0,
-                         "slow": 1.0})
+            rot_scaling={"factor": 4.0, "original": 4096, "fast": 16.0,
+                         "slow": 2.0})
 
         def attn(src=None):
             return MaskedAttentionConfig(

@@ -373,11 +373,11 @@ def test_config_reader_rejects_bad_borrowing():
 @pytest.mark.parametrize("layers,kw", [
     ([(O.latent_mixer(heads=4, dim=32, rot_dim=32, vdim=32, kv_rank=64,
                       scaling=YARN), O.dense_mlp(256)),
-      (O.window_mixer(heads=8, kv_heads=2, dim=64, vdim=32, window=40,
-                      conv=3), O.moe_mlp(experts=8, top=2, ff=64, groups=2,
+      (O.window_mixer(heads=8, kv_heads=2, dim=64, vdim=32, window=44,
+                      conv=4), O.moe_mlp(experts=8, top=2, ff=64, groups=2,
                                          keep=1, shared_ff=96)),
       (O.window_mixer(heads=4, kv_heads=2, dim=64, vdim=32, window=24,
-                      conv=3, kv_from=1), O.moe_mlp(experts=8, top=3, ff=32,
+                      conv=4, kv_from=1), O.moe_mlp(experts=8, top=3, ff=32,
                                                     groups=4, keep=2,
                                                     shared_ff=32))],
      dict(width=128, side_dim=16)),

@@ -14,6 +14,7 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 import lelitar_oracle as O  # noqa: E402
 import pekarax_oracle as PO  # noqa: E402
+import sipelorn_oracle as SO  # noqa: E402
 import volalorn_oracle as VO  # noqa: E402
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -47,8 +48,25 @@ def _pekarax_case():
     return PO, cfg, PO.random_weights(cfg, seed=23)
 
 
+class _SipelornOracle:
+    """The Sipelorn oracle behind the other oracles' call signature."""
+    save_checkpoint = staticmethod(SO.save_checkpoint)
+
+    @staticmethod
+    def forward(cfg, w, tokens):
+        return SO.forward(tokens, w, cfg).float()
+
+
+def _sipelorn_case():
+    cfg = SO.make_config(
+        [(SO.latent_mixer(), SO.moe_mlp()),
+         (SO.window_mixer(window=6), SO.dense_mlp()),
+         (SO.window_mixer(window=9, kv_from=1), None)], vocab=120)
+    return _SipelornOracle, cfg, SO.random_weights(cfg, seed=24)
+
+
 @pytest.mark.parametrize("case", [_lelitar_case, _volalorn_case,
-                                  _pekarax_case])
+                                  _pekarax_case, _sipelorn_case])
 def test_trace_run_mixed_steps_match_oracle(tmp_path, case):
     O, cfg, w = case()
     model = str(tmp_path / "ckpt")
