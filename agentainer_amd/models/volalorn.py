@@ -323,7 +323,8 @@ class MaskedAttention(torch.nn.Module):
             k = qkv[:, k0:v0].view(T, G, mc.dim)
             v = qkv[:, v0:c_end].view(T, G, mc.vdim)
             if mc.plain_qk:
-                ops.kv_append(k, v, k_cache, v_cache, md.slot_mapping)
+                ops.head_kv_append(k, v, k_cache, v_cache,
+                                   md.slot_mapping)
             else:
                 ops.rotary_norm_append(q, k, v, k_cache, v_cache, cos_sin,
                                        md.slot_mapping, self.eps, self.q_norm,

@@ -947,12 +947,12 @@ def latent_rotary_append(proj, heads: int, q_head: int, q_rot_off: int,
                                        cache, slot_mapping)
 
 
-def kv_append(k, v, k_cache, v_cache, slot_mapping):
-    mod = _dispatch_gated("kv_append", k)
+def head_kv_append(k, v, k_cache, v_cache, slot_mapping):
+    mod = _dispatch_gated("head_kv_append", k)
     if mod:
-        mod.kv_append(k, v, k_cache, v_cache, slot_mapping)
+        mod.head_kv_append(k, v, k_cache, v_cache, slot_mapping)
     else:
-        reference.kv_append(k, v, k_cache, v_cache, slot_mapping)
+        reference.head_kv_append(k, v, k_cache, v_cache, slot_mapping)
 
 
 def sigmoid_gate_rows(out, a, gate):

@@ -26,7 +26,7 @@ void latent_rotary_append(torch::Tensor proj, long heads, long q_head,
                           long rot_dim, torch::Tensor w_kv, double eps,
                           torch::Tensor cos_sin, torch::Tensor cache,
                           torch::Tensor slot_mapping);
-void kv_append(torch::Tensor k, torch::Tensor v, torch::Tensor k_cache,
+void head_kv_append(torch::Tensor k, torch::Tensor v, torch::Tensor k_cache,
                torch::Tensor v_cache, torch::Tensor slot_mapping);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -45,5 +45,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "stacked SiLU-gated experts times routing weight, with a tail expert");
   m.def("latent_rotary_append", &latent_rotary_append,
         "rotate query parts, norm the latent, append latent | rotated key");
-  m.def("kv_append", &kv_append, "copy K/V rows into the per-head pools");
+  m.def("head_kv_append", &head_kv_append, "copy K/V rows into the per-head pools");
 }

@@ -14,7 +14,7 @@
 //   coordinates from 2*half on pass unchanged; cos_sin [T, 2*half] fp32 is
 //   the step's cos | sin table. All math fp32. slot < 0 skips the append.
 //
-//   kv_append: k [T, G, D], v [T, G, Dv] copied to the per-head pools
+//   head_kv_append: k [T, G, D], v [T, G, Dv] copied to the per-head pools
 //   [P, G, PS, D] / [P, G, PS, Dv] at slot = page*PS + offset.
 
 #include <torch/extension.h>
@@ -124,7 +124,7 @@ void latent_rotary_append(torch::Tensor proj, long heads, long q_head,
   });
 }
 
-void kv_append(torch::Tensor k, torch::Tensor v, torch::Tensor k_cache,
+void head_kv_append(torch::Tensor k, torch::Tensor v, torch::Tensor k_cache,
                torch::Tensor v_cache, torch::Tensor slot_mapping) {
   TORCH_CHECK(k.dim() == 3 && v.dim() == 3 && k.stride(2) == 1 &&
               v.stride(2) == 1 && k.size(0) == v.size(0) &&

@@ -899,7 +899,7 @@ def latent_rotary_append(proj: torch.Tensor, heads: int, q_head: int,
         flat[rows, kv_rank + rot_dim:] = 0
 
 
-def kv_append(k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
+def head_kv_append(k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
               v_cache: torch.Tensor, slot_mapping: torch.Tensor) -> None:
     """k [T, G, D], v [T, G, Dv] -> pools [P, G, PS, D] / [P, G, PS, Dv] at
     slot = page*PS + offset (slot < 0 skips)."""

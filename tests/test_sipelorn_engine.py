@@ -393,6 +393,14 @@ def test_bf16_serving_path_close_to_oracle(tmp_path, layers, kw):
     step after step."""
     cfg = O.make_config(layers, vocab=300, **kw)
     w = O.random_weights(cfg, seed=11)
+    for k in w:
+        # With random corrections about one token in ten picks its experts
+        # by less than bf16 rounding of the scores, takes other experts than
+        # the oracle, and disturbs the tokens that read it through a
+        # convolution or a window. The choice itself is tested in fp32; here
+        # corrections two apart fix it (the weights still vary by token).
+        if k.endswith("mlp.correction"):
+            w[k] = -2.0 * torch.arange(w[k].numel(), dtype=torch.float32)
     eng, inst, _ = make_instance(tmp_path, cfg, w, "cuda", dtype="bfloat16",
                                  page=16, pool_tokens=512)
     reqs = {"a": tokens_for(cfg, 120, 1), "b": tokens_for(cfg, 75, 2)}
@@ -405,7 +413,5 @@ def test_bf16_serving_path_close_to_oracle(tmp_path, layers, kw):
         d = got[i] - want
         d = d - d.mean(-1, keepdim=True)
         rel = d.pow(2).mean(-1).sqrt() / want.pow(2).mean().sqrt()
-        # a position where two experts score within bf16 rounding of each
-        # other may take the other one; its neighbours do not
-        assert int((rel > 0.08).sum()) <= 0.05 * rel.numel(), rel
+        assert float(rel.max()) < 0.08, rel
         assert float(rel.median()) < 0.03, float(rel.median())

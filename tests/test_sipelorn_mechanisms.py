@@ -333,7 +333,7 @@ def test_plain_kv_append_into_pages(device):
     kc = torch.zeros(5, G, PS, D, device=device)
     vc = torch.zeros(5, G, PS, Dv, device=device)
     slots = torch.tensor([4, 5, 6, 7, 16, -1, 3], device=device)
-    ops.kv_append(k.to(device)[:, :G * D].view(T, G, D),
+    ops.head_kv_append(k.to(device)[:, :G * D].view(T, G, D),
                   v.to(device).view(T, G, Dv), kc, vc, slots)
     for t, s in enumerate(slots.tolist()):
         if s < 0:
