@@ -336,13 +336,10 @@ class MaskedAttention(torch.nn.Module):
             md.query_lens if md.is_prefill else None,
             mc.scale, mc.mask_kind, mc.mask_size, mc.keep_first,
             mc.sigmoid_weights, mc.softcap, self.key_bias,
-            proj[:, g0:g0 + H] if mc.head_gate else None,
+            proj[:, g0:g0 + self.gate_sz] if self.gate_sz else None,
             max_qlen=md.max_qlen if md.is_prefill else 1,
             dist_bias=self.dist_bias)
-        out = out.view(T, H * mc.vdim)
-        if mc.elem_gate:
-            ops.sigmoid_gate_rows(out, out, proj[:, g0:g0 + self.gate_sz])
-        y = ops.linear(out, self.w_o)
+        y = ops.linear(out.view(T, H * mc.vdim), self.w_o)
         if self.extra_rows:
             return y, proj[:, self.extra_off:self.extra_off + self.extra_rows]
         return y

@@ -11,7 +11,9 @@
 //            chunk    j <= p and floor(p/size) == floor(j/size)
 //   weight : softmax over the visible keys, or sigmoid(score + bias[h])
 //            per visible key with no normalization
-//   out    = sum_j weight_j v_j  (* sigmoid(gate[t, h]) when a gate is given)
+//   out    = sum_j weight_j v_j  (* sigmoid(gate[t, h]) when a gate is given;
+//            a gate of heads * Dv columns gates every output coordinate:
+//            * sigmoid(gate[t, h * Dv + e]))
 //
 // Every query therefore sees at most two key ranges: a kept prefix [0, ns)
 // and a main range [lo, p]. Scores, masks, weights and accumulation are
@@ -113,8 +115,8 @@ __global__ __launch_bounds__(64) void masked_attn_rowwave_kernel(
     const int* __restrict__ q_starts, const int* __restrict__ q_lens,
     float scale, int kind, int size, int keep, int sigmoid_w, float softcap,
     const float* __restrict__ key_bias, const T* __restrict__ gate, long g_ts,
-    const float* __restrict__ dist, int H, int G, int D, int Dv, int PS,
-    int max_pages, int vec) {
+    int gate_elem, const float* __restrict__ dist, int H, int G, int D, int Dv,
+    int PS, int max_pages, int vec) {
   extern __shared__ float smem[];
   float* q_s = smem;       // [D]
   float* p_s = smem + D;   // [64]
@@ -199,11 +201,17 @@ __global__ __launch_bounds__(64) void masked_attn_rowwave_kernel(
     __syncthreads();
   }
   float mul = sigmoid_w ? 1.0f : 1.0f / l;
-  if (gate != nullptr) mul *= sigmoidf_(ldf(gate, rowi * g_ts + h));
+  if (gate != nullptr && !gate_elem)
+    mul *= sigmoidf_(ldf(gate, rowi * g_ts + h));
 #pragma unroll
   for (int k = 0; k < RW_MAX_ACC; ++k) {
     const int d = k * WAVE + lane;
-    if (d < Dv) stf(op, d, acc[k] * mul);
+    if (d < Dv) {
+      float o = acc[k] * mul;
+      if (gate != nullptr && gate_elem)
+        o *= sigmoidf_(ldf(gate, rowi * g_ts + (long)h * Dv + d));
+      stf(op, d, o);
+    }
   }
 }
 
@@ -232,8 +240,9 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
     const int* __restrict__ seq_lens, const int* __restrict__ q_starts,
     const int* __restrict__ q_lens, float scale, int kind, int size, int keep,
     int sigmoid_w, float softcap, const float* __restrict__ key_bias,
-    const short* __restrict__ gate, long g_ts, const float* __restrict__ dist,
-    int H, int G, int nd, int nv, int PS, int max_pages, int ps_shift) {
+    const short* __restrict__ gate, long g_ts, int gate_elem,
+    const float* __restrict__ dist, int H, int G, int nd, int nv, int PS,
+    int max_pages, int ps_shift) {
   extern __shared__ __attribute__((aligned(16))) short lds[];
   constexpr int KL = NDB / 2;              // 16-byte K loads per thread
   const int D = nd * 32, Dv = nv * 16;
@@ -452,15 +461,22 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
   // ---- epilogue: lane holds O^T[i*16 + lg*4 + r][column]
   if (!col_ok) return;
   float mul = sigmoid_w ? 1.0f : 1.0f / l;
-  if (gate != nullptr)
+  if (gate != nullptr && !gate_elem)
     mul *= sigmoidf_(bits2f(gate[(row_base + qi) * g_ts + h]));
+  const short* ge = (gate != nullptr && gate_elem)
+                        ? gate + (row_base + qi) * g_ts + (long)h * (nv * 16)
+                        : nullptr;
   short* op = out + (row_base + qi) * o_ts + (long)h * o_hs;
 #pragma unroll
   for (int i = 0; i < NVB; ++i) {
     if (i < nv) {
       bf16x4 t;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) t[r] = f2bits(o[i][r] * mul);
+      for (int r = 0; r < 4; ++r) {
+        float v = o[i][r] * mul;
+        if (ge) v *= sigmoidf_(bits2f(ge[i * 16 + lg * 4 + r]));
+        t[r] = f2bits(v);
+      }
       *reinterpret_cast<bf16x4*>(op + i * 16 + lg * 4) = t;
     }
   }
@@ -495,9 +511,10 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
     const short* __restrict__ vc, const int* __restrict__ page_table,
     const int* __restrict__ seq_lens, float scale, int kind, int size, int keep,
     int sigmoid_w, float softcap, const float* __restrict__ key_bias,
-    const short* __restrict__ gate, long g_ts, const float* __restrict__ dist,
-    int H, int G, int nd, int nv, int PS, int max_pages, int ps_shift,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits) {
+    const short* __restrict__ gate, long g_ts, int gate_elem,
+    const float* __restrict__ dist, int H, int G, int nd, int nv, int PS,
+    int max_pages, int ps_shift, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int n_splits) {
   extern __shared__ __attribute__((aligned(16))) short lds[];
   const int D = nd * 32, Dv = nv * 16;
   const int split = blockIdx.x, b = blockIdx.y, g = blockIdx.z;
@@ -735,7 +752,9 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
     if (n_splits == 1) {
       float mul = sigmoid_w ? 1.0f : 1.0f / L;
       if (gate != nullptr)
-        mul *= sigmoidf_(bits2f(gate[(long)b * g_ts + g * R + c]));
+        mul *= sigmoidf_(bits2f(
+            gate[(long)b * g_ts +
+                 (gate_elem ? (long)(g * R + c) * Dv + e : (long)(g * R + c))]));
       out[(long)b * o_ts + (long)(g * R + c) * o_hs + e] = f2bits(O * mul);
     } else {
       part_o[(part_base + c) * Dv + e] = O;
@@ -751,8 +770,8 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
 __global__ __launch_bounds__(64) void masked_attn_combine_kernel(
     short* __restrict__ out, long o_ts, long o_hs,
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
-    const short* __restrict__ gate, long g_ts, int sigmoid_w, int H, int G,
-    int Dv, int n_splits) {
+    const short* __restrict__ gate, long g_ts, int gate_elem, int sigmoid_w,
+    int H, int G, int Dv, int n_splits) {
   const int b = blockIdx.x, h = blockIdx.y;
   const int R = H / G, g = h / R, c = h % R;
   const long base = (long)(b * G + g) * n_splits;
@@ -766,7 +785,8 @@ __global__ __launch_bounds__(64) void masked_attn_combine_kernel(
     L = fmaf(part_ml[((base + s) * R + c) * 2 + 1], f, L);
   }
   float mul = sigmoid_w ? 1.0f : (L > 0.f ? 1.0f / L : 0.f);
-  if (gate != nullptr) mul *= sigmoidf_(bits2f(gate[(long)b * g_ts + h]));
+  if (gate != nullptr && !gate_elem)
+    mul *= sigmoidf_(bits2f(gate[(long)b * g_ts + h]));
   for (int e = threadIdx.x; e < Dv; e += WAVE) {
     float O = 0.f;
     for (int s = 0; s < n_splits; ++s) {
@@ -774,6 +794,8 @@ __global__ __launch_bounds__(64) void masked_attn_combine_kernel(
           sigmoid_w ? 1.0f : expf(part_ml[((base + s) * R + c) * 2] - M);
       O = fmaf(part_o[((base + s) * R + c) * Dv + e], f, O);
     }
+    if (gate != nullptr && gate_elem)
+      O *= sigmoidf_(bits2f(gate[(long)b * g_ts + (long)h * Dv + e]));
     out[(long)b * o_ts + (long)h * o_hs + e] = f2bits(O * mul);
   }
 }
@@ -839,11 +861,16 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
     kb = key_bias->data_ptr<float>();
   }
   long g_ts = 0;
+  int gate_elem = 0;   // 1: the gate has one column per output coordinate
   if (head_gate.has_value()) {
     TORCH_CHECK(head_gate->dim() == 2 && head_gate->size(0) == T_ &&
-                head_gate->size(1) == H && head_gate->stride(1) == 1 &&
-                head_gate->scalar_type() == q.scalar_type());
+                (head_gate->size(1) == H ||
+                 head_gate->size(1) == (long)H * Dv) &&
+                head_gate->stride(1) == 1 &&
+                head_gate->scalar_type() == q.scalar_type(),
+                "gate is [tokens, heads] or [tokens, heads * value size]");
     g_ts = head_gate->stride(0);
+    gate_elem = head_gate->size(1) != H ? 1 : 0;
   }
   const float* db = nullptr;
   if (dist_bias.has_value()) {
@@ -900,8 +927,8 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                      page_table.data_ptr<int>(), seq_lens.data_ptr<int>(),    \
                      (float)scale, (int)mask_kind, (int)mask_size, keep,      \
                      sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts,   \
-                     db, H, G, nd, nv, PS, max_pages, ps_shift, pop, pmlp,    \
-                     (int)n_splits)
+                     gate_elem, db, H, G, nd, nv, PS, max_pages, ps_shift,    \
+                     pop, pmlp, (int)n_splits)
       if (nd <= 4 && nv <= 4) {
         LAUNCH_DECODE(4, 4);
       } else if (nd <= 4 && nv <= 8) {
@@ -913,7 +940,7 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
       if (n_splits > 1) {
         hipLaunchKernelGGL(masked_attn_combine_kernel, dim3(B, H), dim3(64), 0,
                            stream, (short*)out.data_ptr(), (long)out.stride(0),
-                           (long)out.stride(1), pop, pmlp, gp, g_ts,
+                           (long)out.stride(1), pop, pmlp, gp, g_ts, gate_elem,
                            sigmoid_weights ? 1 : 0, H, G, Dv, (int)n_splits);
       }
       return;
@@ -931,7 +958,7 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                      page_table.data_ptr<int>(), seq_lens.data_ptr<int>(), qs, \
                      ql, (float)scale, (int)mask_kind, (int)mask_size, keep,  \
                      sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts,   \
-                     db, H, G, nd, nv, PS, max_pages, ps_shift)
+                     gate_elem, db, H, G, nd, nv, PS, max_pages, ps_shift)
     if (nd <= 4 && nv <= 4) {
       LAUNCH_MFMA(4, 4);
     } else if (nd <= 4 && nv <= 8) {
@@ -958,7 +985,7 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
         (const T*)k_cache.data_ptr(), (const T*)v_cache.data_ptr(),
         page_table.data_ptr<int>(), seq_lens.data_ptr<int>(), qs, ql,
         (float)scale, (int)mask_kind, (int)mask_size, keep,
-        sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts, db, H, G, D, Dv,
-        PS, max_pages, vec);
+        sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts, gate_elem, db, H,
+        G, D, Dv, PS, max_pages, vec);
   });
 }

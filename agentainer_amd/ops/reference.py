@@ -467,7 +467,8 @@ def masked_attention(out: torch.Tensor, q: torch.Tensor,
     softcap > 0. Weights are a softmax over the visible keys, or (with
     sigmoid_weights) sigmoid(score + key_bias[h]) per visible key without
     normalization. head_gate [T, H], when given, multiplies head h's
-    output by sigmoid(head_gate[t, h]). query_starts/query_lens None means
+    output by sigmoid(head_gate[t, h]); with H * Dv columns it gates every
+    output coordinate. query_starts/query_lens None means
     one new token per sequence; rows with seq_len <= 0 come back zero.
     dist_bias fp32 [H, 2] = (r1, r2) per head takes r1 * ln(1 + r2 * (p - j))
     off the (capped) score of key j for the query at position p."""
@@ -507,8 +508,10 @@ def masked_attention(out: torch.Tensor, q: torch.Tensor,
             p = torch.softmax(s.masked_fill(~seen, float("-inf")), dim=-1)
         o = torch.einsum("hqn,nhe->qhe", p, V)
         if head_gate is not None:
-            o = o * torch.sigmoid(head_gate[start:start + qlen].float()
-                                  ).unsqueeze(-1)
+            gt = torch.sigmoid(head_gate[start:start + qlen].float())
+            # [q, H]: one gate per head; [q, H * Dv]: one per coordinate
+            o = o * (gt.unsqueeze(-1) if gt.size(1) == H
+                     else gt.view(qlen, H, -1))
         out[start:start + qlen] = o.to(out.dtype)
 
 

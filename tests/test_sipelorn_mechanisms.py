@@ -316,14 +316,24 @@ def test_window_attention_with_distance_bias(device, dtype, H, G, D, Dv, size,
             torch.tensor([i + 1], **i32), None, None, D ** -0.5,
             ops.MASK_WINDOW, size, dist_bias=dist)
         close(o1[0], want[i], dtype, 2e-5)
-    # the whole sequence as one prompt, first tokens included
+    # the whole sequence as one prompt, first tokens included, with a gate
+    # per output coordinate (columns of a wider projection)
+    gate = rnd(n, H * Dv + 8, seed=6, scale=2.0).to(dtype)
+    gated = want * torch.sigmoid(gate[:, :H * Dv].double()).view(n, H, Dv)
     out = torch.empty(n, H, Dv, device=device, dtype=dtype)
     ops.masked_attention(
         out, q.to(device=device, dtype=dtype), kc, vc, table,
         torch.tensor([n], **i32), torch.tensor([0], **i32),
         torch.tensor([n], **i32), D ** -0.5, ops.MASK_WINDOW, size,
-        max_qlen=n, dist_bias=dist)
-    close(out, want, dtype, 2e-5)
+        head_gate=gate.to(device)[:, :H * Dv], max_qlen=n, dist_bias=dist)
+    close(out, gated, dtype, 2e-5)
+    i = n - 1                                   # and decoded
+    o1 = torch.empty(1, H, Dv, device=device, dtype=dtype)
+    ops.masked_attention(
+        o1, q[i:i + 1].to(device=device, dtype=dtype), kc, vc, table,
+        torch.tensor([n], **i32), None, None, D ** -0.5, ops.MASK_WINDOW,
+        size, head_gate=gate.to(device)[i:i + 1, :H * Dv], dist_bias=dist)
+    close(o1[0], gated[i], dtype, 2e-5)
 
 
 @pytest.mark.parametrize("device", DEVICES)
